@@ -1,8 +1,8 @@
 """Typed configurations and the one registry from an architecture's name to
 its configuration class and model builder.
 
-config.json names its architecture twice: ``architectures[0]`` (a class name)
-and ``model_type``.  Both are registered; lookup prefers the first.  The
+config.json names its architecture as ``architectures[0]`` (a class name),
+``model_type`` or ``architecture``.  All are looked up, in this order.  The
 reference has no registry, only a ``model_type == 'llama'`` check
 (runtime/checkpoint.py:12).
 """
@@ -47,7 +47,7 @@ def registered_architectures():
 
 def architecture_of(raw):
     """The registry entry for a config.json dict."""
-    candidates = list(raw.get("architectures") or []) + [raw.get("model_type")]
+    candidates = list(raw.get("architectures") or []) + [raw.get("model_type"), raw.get("architecture")]
     for name in candidates:
         if name in _REGISTRY:
             return _REGISTRY[name]

@@ -1,0 +1,169 @@
+// Row-wise kernels of layers that norm a sublayer's output before the residual sum, of feed-forwards with a
+// clamped gate, and of attention that norms its queries and keys per head and gates its heads:
+//   x += mult * rmsnorm(y) * w                      (also with y = (rmsnorm(a) wa + rmsnorm(b) wb) / 2 made on the way)
+//   act = g sigmoid(slope g) (u + shift), g = min(gate, limit), u = clamp(up, -limit, limit)
+//   q, k normed per head, q into a buffer of padded heads, k and v into the pages of the cache
+//   out[t, h, :] = attn[t, h, :vdim] * sigmoid(gate[t, h])
+// Statistics and the residual stream are float; `T` is the storage type of activations (float or bf16).
+#include "common.h"
+
+// ------------------------------------------------- norm of a sublayer's output, scaled, into the residual stream
+// One block a row.  TWO: the row is half the sum of two rows, each normed over the width with a weight of its own.
+// A row is read three times (its squares, the squares of what is normed, the sum): the second and third from cache.
+template <bool TWO>
+__global__ void __launch_bounds__(256)
+post_norm_add_kernel(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ wa,
+                     const float* __restrict__ b, const float* __restrict__ wb, const float* __restrict__ w,
+                     int dim, float eps, float mult) {
+    __shared__ float red[4];
+    const size_t row = blockIdx.x;
+    const float* ar = a + row * dim;
+    const float* br = TWO ? b + row * dim : nullptr;
+    float sa = 0.f, sb = 0.f;
+    for (int d = threadIdx.x; d < dim; d += 256) {
+        const float u = ar[d];
+        sa += u * u;
+        if (TWO) { const float v = br[d]; sb += v * v; }
+    }
+    float ra = 1.f, rb = 0.f;
+    if (TWO) {
+        ra = 0.5f / sqrtf(block_sum<256>(sa, red) / (float)dim + eps);
+        rb = 0.5f / sqrtf(block_sum<256>(sb, red) / (float)dim + eps);
+        sa = 0.f;
+        for (int d = threadIdx.x; d < dim; d += 256) {
+            const float y = ar[d] * ra * wa[d] + br[d] * rb * wb[d];
+            sa += y * y;
+        }
+    }
+    // (w null: the row is added as it is, times mult)
+    const float scale = w ? mult / sqrtf(block_sum<256>(sa, red) / (float)dim + eps) : mult;
+    float* xr = x + row * dim;
+    for (int d = threadIdx.x; d < dim; d += 256) {
+        const float y = TWO ? ar[d] * ra * wa[d] + br[d] * rb * wb[d] : ar[d];
+        xr[d] += y * scale * (w ? w[d] : 1.0f);
+    }
+}
+
+extern "C" int cisr_post_norm_add(float* x, const float* a, const float* wa, const float* b, const float* wb,
+                                  const float* w, int rows, int dim, float eps, float mult, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (dim <= 0 || (b != nullptr && (wa == nullptr || wb == nullptr))) return (int)hipErrorInvalidValue;
+    if (b) post_norm_add_kernel<true><<<rows, 256, 0, stream>>>(x, a, wa, b, wb, w, dim, eps, mult);
+    else post_norm_add_kernel<false><<<rows, 256, 0, stream>>>(x, a, nullptr, nullptr, nullptr, w, dim, eps, mult);
+    return CISR_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------ clamped gated activation
+// gu[r] = [gate (inter) | up (inter)]; arithmetic in float.
+template <typename T>
+__global__ void glu_clamped_kernel(const T* __restrict__ gu, T* __restrict__ act, int inter, size_t n,
+                                   float limit, float slope, float shift) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const size_t row = i / inter;
+    const int col = (int)(i % inter);
+    const T* base = gu + row * (size_t)(2 * inter);
+    const float g = fminf(load_f32(base + col), limit);
+    const float u = fminf(fmaxf(load_f32(base + inter + col), -limit), limit);
+    store_f32(act + i, g / (1.0f + expf(-slope * g)) * (u + shift));
+}
+
+extern "C" int cisr_glu_clamped(const void* gu, void* act, int rows, int inter, float limit, float slope, float shift,
+                                int dtype, hipStream_t stream) {
+    const size_t n = (size_t)rows * inter;
+    if (n == 0) return 0;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (dtype == DT_F32) glu_clamped_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)act, inter, n, limit, slope, shift);
+    else glu_clamped_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)act, inter, n, limit, slope, shift);
+    return CISR_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------- per-head norm of queries and keys + scatter into the pages
+// One block a token row, a wave a head at a time.  The row of the fused projection is [q: heads x dim |
+// k: kv_heads x dim | v: kv_heads x vdim | ...].  Queries go to q_out [T, heads, pad] (coordinates dim..pad-1 zero),
+// keys to kcache [pages, kv_heads, page_size, pad] (likewise), values transposed to vcache [pages, kv_heads, pad,
+// page_size] (coordinates vdim..pad-1 zero): heads of `pad` coordinates are what the attention kernels read.
+// wq / wk null: that side is not normed.
+template <typename T>
+__global__ void __launch_bounds__(256)
+qk_norm_scatter_kernel(const T* __restrict__ qkv, int ld, const float* __restrict__ wq, const float* __restrict__ wk,
+                       T* __restrict__ q_out, T* __restrict__ kcache, T* __restrict__ vcache,
+                       const int* __restrict__ slots, int heads, int kv_heads, int dim, int vdim, int pad,
+                       int page_size, float eps) {
+    const int row = blockIdx.x, wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    const T* src = qkv + (size_t)row * ld;
+    const int slot = slots ? slots[row] : -1;
+    const int items = heads + 2 * kv_heads;
+    for (int item = wave; item < items; item += 4) {
+        if (item < heads + kv_heads) {
+            const bool is_q = item < heads;
+            const int head = is_q ? item : item - heads;
+            if (!is_q && slot < 0) continue;
+            const T* v = src + (size_t)item * dim;         // (queries and keys have the same size: one run of heads)
+            const float* w = is_q ? wq : wk;
+            float vals[4], ss = 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int d = lane + WAVE * i;
+                vals[i] = d < dim ? load_f32(v + d) : 0.f;
+                ss += vals[i] * vals[i];
+            }
+            const float scale = w ? 1.0f / sqrtf(wave_sum(ss) / (float)dim + eps) : 1.0f;
+            T* dst = is_q ? q_out + ((size_t)row * heads + head) * pad
+                          : kcache + (((size_t)(slot / page_size) * kv_heads + head) * page_size + slot % page_size) * pad;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int d = lane + WAVE * i;
+                if (d < pad) store_f32(dst + d, d < dim ? vals[i] * scale * (w ? w[d] : 1.0f) : 0.f);
+            }
+        } else {
+            if (slot < 0) continue;
+            const int head = item - heads - kv_heads;
+            const T* v = src + (size_t)(heads + kv_heads) * dim + (size_t)head * vdim;
+            T* dst = vcache + ((size_t)(slot / page_size) * kv_heads + head) * pad * page_size + slot % page_size;
+            for (int d = lane; d < pad; d += WAVE) store_f32(dst + (size_t)d * page_size, d < vdim ? load_f32(v + d) : 0.f);
+        }
+    }
+}
+
+extern "C" int cisr_qk_norm_scatter(const void* qkv, int ld, const float* wq, const float* wk, void* q_out, void* kcache,
+                                    void* vcache, const int* slots, int rows, int heads, int kv_heads, int dim, int vdim,
+                                    int pad, int page_size, float eps, int dtype, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (dim <= 0 || vdim <= 0 || dim > pad || vdim > pad || pad > 256 || page_size <= 0 ||
+        ld < (heads + kv_heads) * dim + kv_heads * vdim)
+        return (int)hipErrorInvalidValue;
+    if (dtype == DT_F32)
+        qk_norm_scatter_kernel<float><<<rows, 256, 0, stream>>>((const float*)qkv, ld, wq, wk, (float*)q_out, (float*)kcache,
+            (float*)vcache, slots, heads, kv_heads, dim, vdim, pad, page_size, eps);
+    else
+        qk_norm_scatter_kernel<bf16_t><<<rows, 256, 0, stream>>>((const bf16_t*)qkv, ld, wq, wk, (bf16_t*)q_out, (bf16_t*)kcache,
+            (bf16_t*)vcache, slots, heads, kv_heads, dim, vdim, pad, page_size, eps);
+    return CISR_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------ one gate a head
+// out[t, h, d] = attn[t, h, d] * sigmoid(gate[t * ld_gate + h]) for d < vdim; attn has heads of `pad` coordinates.
+template <typename T>
+__global__ void head_gate_kernel(const T* __restrict__ attn, const T* __restrict__ gate, int ld_gate,
+                                 T* __restrict__ out, int heads, int vdim, int pad, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const int d = (int)(i % vdim);
+    const size_t th = i / vdim;
+    const int h = (int)(th % heads);
+    const size_t t = th / heads;
+    const float g = gate ? 1.0f / (1.0f + expf(-load_f32(gate + t * ld_gate + h))) : 1.0f;
+    store_f32(out + i, load_f32(attn + th * pad + d) * g);
+}
+
+extern "C" int cisr_head_gate(const void* attn, const void* gate, int ld_gate, void* out, int rows, int heads, int vdim,
+                              int pad, int dtype, hipStream_t stream) {
+    const size_t n = (size_t)rows * heads * vdim;
+    if (n == 0) return 0;
+    if (vdim > pad) return (int)hipErrorInvalidValue;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (dtype == DT_F32) head_gate_kernel<float><<<blocks, 256, 0, stream>>>((const float*)attn, (const float*)gate, ld_gate, (float*)out, heads, vdim, pad, n);
+    else head_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)attn, (const bf16_t*)gate, ld_gate, (bf16_t*)out, heads, vdim, pad, n);
+    return CISR_LAUNCH_CHECK();
+}

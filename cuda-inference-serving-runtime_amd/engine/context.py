@@ -70,6 +70,7 @@ class StepContext:
         # part that was told it may (`next_norm`), taken by the norm that reads the rows next (or settled)
         self.unfinished = None
         self.next_norm = None     # the norm that reads the residual stream after the block that runs now, if known
+        self.layer_tap = getattr(runner, "layer_tap", None)   # callable(schedule index, residual rows) after every layer run, or None
         self.capturing = False    # the step is being recorded into a graph: launches only
         self.owner = None         # key of the captured program this step belongs to, if any
 

@@ -71,7 +71,7 @@ def random_model(config, seed=0, dtype="bfloat16", device="cuda:0", std=0.02):
     for spec in sorted(model.tensor_specs(), key=lambda s: s.name):
         if spec.integer:
             raise ValueError(f"{spec.name}: integer tables have no random initialisation")
-        values = torch.randn(spec.shape, generator=generator, device=device, dtype=torch.float32) * std
+        values = torch.randn(spec.drawn_shape(), generator=generator, device=device, dtype=torch.float32) * std
         if spec.init == "one_plus_normal":
             values += 1.0
         tensors[spec.name] = values.to(torch.bfloat16 if dtype == torch.bfloat16 else torch.float32)

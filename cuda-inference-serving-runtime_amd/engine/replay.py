@@ -25,7 +25,7 @@ from .loading import import_plugins, load_model
 from .runner import ModelRunner, StepEntry
 
 PAGE_SIZE = 16          # divides 64, so a request rounded up to 64 tokens never holds more than its share
-MAX_LIVE = 4
+MAX_LIVE = 4            # requests that are live at one time: the state slots of the run, used again as requests end
 
 
 def replay(model_dir, dtype, out_dir, max_tokens, lines, page_size=PAGE_SIZE, echo=print, execution="eager"):
@@ -35,7 +35,7 @@ def replay(model_dir, dtype, out_dir, max_tokens, lines, page_size=PAGE_SIZE, ec
     out_dir.mkdir(parents=True, exist_ok=True)
     model = load_model(model_dir, dtype=dtype)
     pages = max(1, -(-int(max_tokens) // page_size))
-    runner = ModelRunner(model, n_pages=pages, page_size=page_size, max_requests=4 * MAX_LIVE, execution=execution)
+    runner = ModelRunner(model, n_pages=pages, page_size=page_size, max_requests=MAX_LIVE, execution=execution)
     for line in lines:
         line = line.strip()
         if not line:

@@ -105,6 +105,7 @@ class ModelRunner:
         self._has_picked = set()
         self._last_wanted = None  # (requests, state slots on the host, state slots on the device) of the last step's logits
         self._failed = set()      # requests whose state a failed step may have changed: they can only be released
+        self.layer_tap = None     # callable(schedule index, residual rows): sees the residual stream after every layer run (eager)
 
     # -- requests -------------------------------------------------------------
     def create(self, request):

@@ -1,8 +1,9 @@
 """Builds and loads the HIP kernel library (gfx950 only).
 
 The sources under ``csrc/`` are compiled with ``hipcc`` into shared objects (the
-core, and one per head size of the matrix-core attention, so that a first call
-compiles only what its model needs) whose file names carry a digest of the
+core, one per head size of the matrix-core attention and one for the mixers
+that keep a state per request, so that a first call compiles only what its
+model needs) whose file names carry a digest of the
 sources and flags, so a stale build is never loaded.  Loading looks for that
 file first and compiles only if it is missing; compilation prints a line per
 file so a first call is visibly alive.
@@ -35,6 +36,8 @@ _libs = {}
 
 CORE = "kernels"                                   # everything but the matrix-core attention and the measurement kernels
 MEASURE = "measure"                                # kernels that only measure the machine; the engine never loads them
+RECURRENCE = "recurrence"                          # mixers with a state per request: scans, short convolutions, their gates
+OWN_UNITS = (MEASURE, RECURRENCE)                  # units of one source file of the same name
 ATTENTION_PADS = (32, 64, 96, 128, 160, 192, 224, 256)
 
 
@@ -53,14 +56,14 @@ def attention_unit(dpad):
 def units():
     """The shared objects the kernels are built into: the core, and one per padded head size of the
     matrix-core attention (a model needs only its own, so a first call compiles only that one)."""
-    return [CORE, MEASURE] + [attention_unit(d) for d in ATTENTION_PADS]
+    return [CORE, *OWN_UNITS] + [attention_unit(d) for d in ATTENTION_PADS]
 
 
 def sources(unit=CORE):
     if unit == CORE:
-        return sorted(p for p in CSRC.glob("*.hip") if not p.name.startswith("attention_mfma_d") and p.stem != MEASURE)
-    if unit == MEASURE:
-        return [CSRC / "measure.hip"]
+        return sorted(p for p in CSRC.glob("*.hip") if not p.name.startswith("attention_mfma_d") and p.stem not in OWN_UNITS)
+    if unit in OWN_UNITS:
+        return [CSRC / f"{unit}.hip"]
     path = CSRC / f"attention_mfma_{unit[len('attn_'):]}.hip"
     if not path.exists():
         raise KernelLibraryError(f"no source for kernel unit {unit}")

@@ -66,6 +66,10 @@ def _declare(h):
         "cisr_qkv_rope_wide": [p, i, p, i, p, i, i, i, p, p, p, p, p, p, i, i, i, i, i, p, C.c_longlong, p],
         "cisr_gemm_merged_bf16": [p, p, i, i, i, p, i, p, i, p, i, i, i, p],
         "cisr_gemm_merged_ok": [i, i, i, i, i],
+        "cisr_post_norm_add": [p, p, p, p, p, p, i, i, f, f, p],
+        "cisr_glu_clamped": [p, p, i, i, f, f, f, i, p],
+        "cisr_qk_norm_scatter": [p, i, p, p, p, p, p, p, i, i, i, i, i, i, i, f, i, p],
+        "cisr_head_gate": [p, p, i, p, i, i, i, i, i, p],
     }
     for name, args in sig.items():
         fn = getattr(h, name)
@@ -818,3 +822,208 @@ def take_tokens(tokens, source, sampled):
     _check(lib().cisr_take_tokens(_dev(tokens, "tokens", torch.int32), _dev(source, "source", torch.int32, (rows,)),
                                   _dev(sampled, "sampled", torch.int32), rows, sampled.numel(), _stream()), "take_tokens")
     return tokens
+
+
+# -- layers that norm a sublayer's output, clamped gates, normed and gated attention ----------------------------------
+
+def post_norm_add(x, y, weight, eps, mult, second=None):
+    """x += mult * rmsnorm(y) * weight, in place (all float, [T, H]).  With `second` = (y2, w1, w2) the row that is
+    normed is (rmsnorm(y) w1 + rmsnorm(y2) w2) / 2: two sublayers side by side.  `weight` None: no outer norm,
+    x += mult * row."""
+    rows, dim = x.shape
+    xp = _dev(x, "x", torch.float32)
+    yp = _dev(y, "y", torch.float32, (rows, dim))
+    wp = None if weight is None else _dev(weight, "weight", torch.float32, (dim,))
+    ap = bp = w2p = None
+    if second is not None:
+        y2, w1, w2 = second
+        bp = _dev(y2, "y2", torch.float32, (rows, dim))
+        ap, w2p = _dev(w1, "w1", torch.float32, (dim,)), _dev(w2, "w2", torch.float32, (dim,))
+    _check(lib().cisr_post_norm_add(xp, yp, ap, bp, w2p, wp, rows, dim, float(eps), float(mult), _stream()), "post_norm_add")
+    return x
+
+
+def glu_clamped(gate_up, out, limit, slope=1.702, shift=1.0):
+    """out[r, i] = g sigmoid(slope g) (u + shift), g = min(gate_up[r, i], limit), u = clamp(gate_up[r, I + i], -limit, limit)."""
+    rows, two_i = gate_up.shape
+    if two_i % 2:
+        raise KernelError("glu_clamped: input width must be even")
+    inter = two_i // 2
+    _check(lib().cisr_glu_clamped(_dev(gate_up, "gate_up"), _dev(out, "out", gate_up.dtype, (rows, inter)), rows, inter,
+                                  float(limit), float(slope), float(shift), _storage(gate_up, "gate_up"), _stream()), "glu_clamped")
+    return out
+
+
+def qk_norm_scatter(qkv, q_norm, k_norm, q_out, kcache, vcache, slots, heads, kv_heads, dim, vdim, pad, page_size, eps):
+    """Rows of a fused projection [q: heads x dim | k: kv_heads x dim | v: kv_heads x vdim | ...]: queries and keys
+    RMS-normed per head (weights float [dim], or None: left as they are), queries into q_out [T, heads * pad], keys and
+    values into the cache at `slots`, all as heads of `pad` coordinates whose rest is zero (keys [pages, kv_heads,
+    page_size, pad], values transposed in a page, [pages, kv_heads, pad, page_size])."""
+    rows, ld = qkv.shape
+    if dim > pad or vdim > pad or pad > 256 or ld < (heads + kv_heads) * dim + kv_heads * vdim:
+        raise KernelError(f"qk_norm_scatter: heads of {dim} / {vdim} do not fit rows of {ld} or pages of {pad}")
+    pages = kcache.shape[0]
+    wq = None if q_norm is None else _dev(q_norm, "q_norm", torch.float32, (dim,))
+    wk = None if k_norm is None else _dev(k_norm, "k_norm", torch.float32, (dim,))
+    _check(lib().cisr_qk_norm_scatter(_dev(qkv, "qkv"), ld, wq, wk, _dev(q_out, "q_out", qkv.dtype, (rows, heads * pad)),
+                                      _dev(kcache, "kcache", qkv.dtype, (pages, kv_heads, page_size, pad)),
+                                      _dev(vcache, "vcache", qkv.dtype, (pages, kv_heads, pad, page_size)),
+                                      _dev(slots, "slots", torch.int32, (rows,)), rows, heads, kv_heads, dim, vdim, pad,
+                                      page_size, float(eps), _storage(qkv, "qkv"), _stream()), "qk_norm_scatter")
+    return q_out
+
+
+def head_gate(attn, gates, out, heads, vdim, pad):
+    """out[t, h, :] = attn[t, h, :vdim] * sigmoid(gates[t, h]); attn [T, heads * pad], gates a view [T, heads] of a
+    row-major buffer (or None: no gate, the heads are only packed), out [T, heads * vdim]."""
+    rows = attn.shape[0]
+    gp, ldg = None, 0
+    if gates is not None:
+        if gates.dtype != attn.dtype or tuple(gates.shape) != (rows, heads) or gates.stride(1) != 1 or not gates.is_cuda:
+            raise KernelError("head_gate: gates must be [T, heads] of the activations' dtype with unit stride")
+        gp, ldg = gates.data_ptr(), gates.stride(0)
+    _check(lib().cisr_head_gate(_dev(attn, "attn", None, (rows, heads * pad)), gp, ldg,
+                                _dev(out, "out", attn.dtype, (rows, heads * vdim)), rows, heads, vdim, pad,
+                                _storage(attn, "attn"), _stream()), "head_gate")
+    return out
+
+
+# -- mixers with a state per request (the kernels of csrc/recurrence.hip, a shared object of their own) ---------------
+
+_recurrence = None
+
+
+def _rec():
+    global _recurrence
+    if _recurrence is None:
+        h = library.load(library.RECURRENCE)
+        p, i, f, ll = C.c_void_p, C.c_int, C.c_float, C.c_longlong
+        sig = {
+            "cisr_linear_scan": [p, i, p, i, p, i, p, i, i, p, i, p, i, p, ll, p, p, i, i, i, i, i, f, i, p],
+            "cisr_conv_silu": [p, i, i, p, p, p, ll, p, p, p, p, i, i, i, i, i, i, p, p, p, p, p],
+            "cisr_decay_gate": [p, i, p, p, i, i, f, p],
+            "cisr_group_norm_gate": [p, p, i, p, i, p, i, p, i, p, i, i, i, f, i, i, p],
+        }
+        for name, args in sig.items():
+            fn = getattr(h, name)
+            fn.argtypes = args
+            fn.restype = C.c_int
+        _recurrence = h
+    return _recurrence
+
+
+def _rows_of(t, name, cols=None):
+    """(pointer, row stride) of a float matrix view with unit column stride."""
+    if not isinstance(t, torch.Tensor) or not t.is_cuda or t.dtype != torch.float32 or t.dim() != 2 or t.stride(1) != 1:
+        raise KernelError(f"{name}: expected a float GPU matrix with contiguous rows")
+    if cols is not None and t.shape[1] != cols:
+        raise KernelError(f"{name}: {t.shape[1]} columns, expected {cols}")
+    return t.data_ptr(), t.stride(0)
+
+
+def scan_columns(segments, heads, cols):
+    """Columns of the state that one wave of the linear scan owns (16, 8 or 4): fewer columns make more waves of the
+    same head, until the launch has about two waves for every SIMD of the GPU."""
+    for width in (16, 8, 4):
+        if segments * heads * -(-cols // width) >= 2048 or width == 4:
+            return width
+
+
+def linear_scan(q, k, v, decay, out, state, seg_start, state_slots, heads, rows_of_state, cols_of_state, share=1,
+                step=None, q_scale=1.0, columns=None):
+    """Per segment and head: S_t = diag(a_t) S_(t-1) + k_t (v_t step_t)^T, o_t = q_scale S_t^T q_t over the segment's
+    rows in order, S [rows_of_state, cols_of_state] read from and written back to the segment's state slot.
+    q, k float views [T, heads / share * R]; v, out [T, heads * C]; decay [T, heads * R] (a vector a head) or
+    [T, heads] (a number a head); step None or [T, heads]; state float [slots, >= heads * R * C] (a view whose rows
+    start with the state); seg_start int32 [S + 1]; state_slots int32 [S]."""
+    R, Cc = int(rows_of_state), int(cols_of_state)
+    T = v.shape[0]
+    segments = state_slots.shape[0]
+    if heads % share or R > 64 * 16:
+        raise KernelError("linear_scan: heads must divide into their groups and a state has at most 1024 rows")
+    qp, ldq = _rows_of(q, "q", heads // share * R)
+    kp, ldk = _rows_of(k, "k", heads // share * R)
+    vp, ldv = _rows_of(v, "v", heads * Cc)
+    op, ldo = _rows_of(out, "out", heads * Cc)
+    if decay.shape[1] not in (heads, heads * R):
+        raise KernelError("linear_scan: decays are one a head or one a state row")
+    vec = decay.shape[1] != heads
+    ap, lda = _rows_of(decay, "decay")
+    sp, lds = (None, 0) if step is None else _rows_of(step, "step", heads)
+    if any(t.shape[0] != T for t in (q, k, decay, out)) or (step is not None and step.shape[0] != T):
+        raise KernelError("linear_scan: operands differ in rows")
+    if state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < heads * R * Cc or not state.is_cuda:
+        raise KernelError("linear_scan: the state must be float [slots, >= heads * R * C]")
+    cols = int(columns or scan_columns(segments, heads, Cc))
+    while -(-R // (64 // cols)) > 64:
+        cols *= 2          # (a lane holds at most 64 rows of its column)
+    _check(_rec().cisr_linear_scan(qp, ldq, kp, ldk, vp, ldv, ap, lda, int(vec), sp, lds, op, ldo, state.data_ptr(),
+                                   state.stride(0), _dev(seg_start, "seg_start", torch.int32, (segments + 1,)),
+                                   _dev(state_slots, "state_slots", torch.int32, (segments,)), segments, heads, R, Cc,
+                                   int(share), float(q_scale), cols, _stream()), "linear_scan")
+    return out
+
+
+def conv_silu(x, taps_weight, bias, conv_state, out, seg_of_row, seg_start, state_slots, gates=None):
+    """out[t, c] = silu(bias[c] + sum_j w[c, j] input(t - (K - 1) + j)[c]) over the rows of each segment, the K - 1 inputs
+    before a segment's first row taken from its state slot, which then moves on to the last K - 1 inputs.
+    x float view [T, channels]; taps_weight float [channels, K]; conv_state float view [slots, >= (K - 1) * channels].
+    `gates` = (dt view [T, heads], dt_bias [heads], a_log [heads], step out [T, heads], decay out [T, heads]):
+    step = softplus(dt + dt_bias), decay = exp(-exp(a_log) step), made by the same launch."""
+    T, channels = x.shape
+    K = taps_weight.shape[1]
+    segments = state_slots.shape[0]
+    xp, ld = _rows_of(x, "x")
+    if conv_state.dtype != torch.float32 or conv_state.stride(1) != 1 or conv_state.shape[1] < (K - 1) * channels:
+        raise KernelError("conv_silu: the state must be float [slots, >= (K - 1) * channels]")
+    heads, dtp, dt_first, bp2, alp, stp, dcp = 0, None, 0, None, None, None, None
+    if gates is not None:
+        dt, dt_bias, a_log, step, decay = gates
+        heads = dt.shape[1]
+        dp, ldd = _rows_of(dt, "dt")
+        if ldd != ld or (dp - xp) % 4:
+            raise KernelError("conv_silu: the step sizes must be columns of the rows that hold the convolution's inputs")
+        dt_first = (dp - xp) // 4
+        bp2, alp = _dev(dt_bias, "dt_bias", torch.float32, (heads,)), _dev(a_log, "a_log", torch.float32, (heads,))
+        stp, dcp = _dev(step, "step", torch.float32, (T, heads)), _dev(decay, "decay", torch.float32, (T, heads))
+    _check(_rec().cisr_conv_silu(xp, ld, 0, _dev(taps_weight, "taps", torch.float32, (channels, K)),
+                                 None if bias is None else _dev(bias, "bias", torch.float32, (channels,)),
+                                 conv_state.data_ptr(), conv_state.stride(0), _dev(out, "out", torch.float32, (T, channels)),
+                                 _dev(seg_of_row, "seg_of_row", torch.int32, (T,)),
+                                 _dev(seg_start, "seg_start", torch.int32, (segments + 1,)),
+                                 _dev(state_slots, "state_slots", torch.int32, (segments,)), T, segments, channels, K, heads,
+                                 dt_first, bp2, alp, stp, dcp, _stream()), "conv_silu")
+    return out
+
+
+def decay_gate(z, bias, out, tau):
+    """out = sigmoid(z + bias)^(1 / tau) in float; z a float view [T, N], bias float [N] or None, out float [T, N]."""
+    T, n = z.shape
+    zp, ld = _rows_of(z, "z")
+    _check(_rec().cisr_decay_gate(zp, ld, None if bias is None else _dev(bias, "bias", torch.float32, (n,)),
+                                  _dev(out, "out", torch.float32, (T, n)), T, n, float(tau), _stream()), "decay_gate")
+    return out
+
+
+def group_norm_gate(y, gate, weight, out, groups, eps, gate_first, shared_weight=False, skip=None):
+    """Rows of y float [T, groups * size] in `groups` equal parts, each divided by its own root mean square, times
+    `weight` ([size] if shared by the parts, else [groups * size]), with silu(gate) multiplied in before the norm
+    (`gate_first`) or after it; `skip` = (d [n], x view [T, groups * size]) adds d[i // (groups * size / n)] x[t, i]
+    first.  gate a float view [T, groups * size]; out [T, groups * size] float or bf16."""
+    T, width = y.shape
+    if width % groups:
+        raise KernelError("group_norm_gate: the row does not divide into its parts")
+    size = width // groups
+    gp, ldg = _rows_of(gate, "gate", width)
+    wp = _dev(weight, "weight", torch.float32, (size if shared_weight else width,))
+    dp, span, xp, ldx = None, 0, None, 0
+    if skip is not None:
+        d, x = skip
+        if width % d.shape[0]:
+            raise KernelError("group_norm_gate: the skip weights do not divide the row")
+        dp, span = _dev(d, "skip", torch.float32), width // d.shape[0]
+        xp, ldx = _rows_of(x, "x", width)
+    _check(_rec().cisr_group_norm_gate(_dev(y, "y", torch.float32), gp, ldg, wp, int(shared_weight), dp, span, xp, ldx,
+                                       _dev(out, "out", None, (T, width)), T, groups, size, float(eps), int(bool(gate_first)),
+                                       _storage(out, "out"), _stream()), "group_norm_gate")
+    return out

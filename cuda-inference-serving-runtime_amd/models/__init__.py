@@ -1,2 +1,3 @@
 from .model import Model, ScheduleEntry
 from .llama import build_llama
+from .novosun import build_novosun

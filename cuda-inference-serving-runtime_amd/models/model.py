@@ -70,7 +70,7 @@ class Model:
         """Names a checkpoint may hold that the model does not read: the copy of a tied head
         (the reference overwrites it with the embedding, runtime/checkpoint.py:38-39)."""
         tied = getattr(self.head, "tied_to", None)
-        return (self.head.name + ".weight",) if tied is not None else ()
+        return (getattr(self.head, "tensor", self.head.name + ".weight"),) if tied is not None else ()
 
     def bind(self, tensors, dtype, device):
         self.dtype, self.device = dtype, device
@@ -126,6 +126,9 @@ class Model:
             following = self.layers[self.schedule[index + 1].layer] if index < last else None
             ctx.next_norm = following.first_norm() if hasattr(following, "first_norm") else None
             x = self.layers[entry.layer].forward(x, ctx, self.site_of(index))
+            if ctx.layer_tap is not None:      # (a caller that looks at the residual stream after every layer run; eager steps only)
+                ctx.settle(x)
+                ctx.layer_tap(index, x)
             ctx.next_norm = None
             if following is None or not hasattr(following, "first_norm"):
                 ctx.settle(x)

@@ -126,4 +126,86 @@ class PagedAttention(Mixer):
         return residual
 
 
+class NormedGatedAttention(Mixer):
+    """Grouped-query softmax attention over the paged cache whose positions do not enter the scores: queries and keys
+    are RMS-normed per head (a weight of size `dim` each, shared by the heads; `qk_norm` False: not normed), the score
+    is (q . k) * scale, keys and values may differ in size (`dim`, `vdim`), and each head's result is multiplied by
+    sigmoid of a projection of the mixer's input, one number a head (`head_gate`).
+
+    The pages hold heads of `pad` = max(dim, vdim) coordinates (rounded up to a multiple of 8), the rest zero: zero
+    coordinates add nothing to a score and give result coordinates that are not read, so the attention kernels
+    of the framework serve as they are.  `names`: the tensors' names under `name` (q, k, v, o, gate, q norm, k norm)."""
+
+    NAMES = {"q": "q", "k": "k", "v": "v", "o": "o", "gate": "g", "q_norm": "q.norm", "k_norm": "k.norm"}
+
+    def __init__(self, name, hidden, heads, kv_heads, dim, vdim, scale, eps, qk_norm=True, head_gate=True, window=None,
+                 names=None, tuning=None):
+        if heads % kv_heads:
+            raise ValueError(f"{heads} query heads are not a multiple of {kv_heads} key/value heads")
+        self.pad = -(-max(dim, vdim) // 8) * 8
+        if self.pad > 256:
+            raise ValueError(f"head sizes {dim} / {vdim}: at most 256")
+        if not scale > 0:
+            raise ValueError("the score scale must be positive")
+        self.name, self.hidden, self.heads, self.kv_heads, self.dim, self.vdim = name, hidden, heads, kv_heads, dim, vdim
+        self.scale, self.eps, self.qk_norm, self.head_gate, self.window = float(scale), float(eps), bool(qk_norm), bool(head_gate), window
+        self.names = {**self.NAMES, **(names or {})}
+        self.tuning = tuning or kernel.DEFAULT_TUNING
+        self.w_in = self.w_out = self.q_weight = self.k_weight = None
+
+    def _tensor(self, which):
+        return f"{self.name}.{self.names[which]}"
+
+    def kernel_units(self, dtype):
+        return kernel.kernel_units(self.pad, dtype)
+
+    def step_arrays(self):
+        return [kernel.SingleRows(self.tuning.split_single_from), kernel.RowsLongestFirst()]
+
+    def cache_need(self):
+        return KVNeed(self.kv_heads, self.pad, self.window)
+
+    def tensor_specs(self):
+        H, nh, nkv, D, V = self.hidden, self.heads, self.kv_heads, self.dim, self.vdim
+        specs = [TensorSpec(self._tensor("q"), (nh * D, H)), TensorSpec(self._tensor("k"), (nkv * D, H)),
+                 TensorSpec(self._tensor("v"), (nkv * V, H)), TensorSpec(self._tensor("o"), (H, nh * V))]
+        if self.head_gate:
+            specs.append(TensorSpec(self._tensor("gate"), (nh, H)))
+        if self.qk_norm:
+            specs += [TensorSpec(self._tensor("q_norm"), (D,), init="one_plus_normal"),
+                      TensorSpec(self._tensor("k_norm"), (D,), init="one_plus_normal")]
+        return specs
+
+    def bind(self, tensors, dtype):
+        parts = [matrix_operand(tensors[self._tensor(p)], dtype) for p in (("q", "k", "v", "gate") if self.head_gate else ("q", "k", "v"))]
+        rows = sum(p.shape[0] for p in parts)
+        if rows % 8:      # rows of the fused projection are a multiple of 16 bytes: zero rows at the end
+            parts.append(torch.zeros(8 - rows % 8, self.hidden, dtype=parts[0].dtype, device=parts[0].device))
+        self.w_in = torch.cat(parts, dim=0).contiguous()
+        self.w_out = matrix_operand(tensors[self._tensor("o")], dtype)
+        if self.qk_norm:
+            self.q_weight = tensors[self._tensor("q_norm")].to(torch.float32).contiguous()
+            self.k_weight = tensors[self._tensor("k_norm")].to(torch.float32).contiguous()
+
+    def output(self, h, ctx, site):
+        """The mixer's result, float [T, hidden], without the residual sum."""
+        T = h.shape[0]
+        nh, nkv, D, V, pad = self.heads, self.kv_heads, self.dim, self.vdim, self.pad
+        gid, kcache, vcache = ctx.cache.pages_of_site(site)
+        view = ctx.kv[gid]
+        qkv = ops.gemm(h, self.w_in, ctx.buffer("gattn.qkv", (T, self.w_in.shape[0]), ctx.dtype), scratch=ctx.scratch)
+        q = ops.qk_norm_scatter(qkv, self.q_weight, self.k_weight, ctx.buffer("gattn.q", (T, nh * pad), ctx.dtype), kcache, vcache,
+                                view.slots, nh, nkv, D, V, pad, view.page_size, self.eps)
+        out = ctx.buffer("gattn.out", (T, nh * pad), ctx.dtype)
+        kernel.paged_attention(ctx, q, nh * pad, kcache, vcache, view, out, nh, nkv, pad, self.window, self.scale, tuning=self.tuning)
+        first_gate = (nh + nkv) * D + nkv * V
+        gates = qkv[:, first_gate:first_gate + nh] if self.head_gate else None
+        act = ops.head_gate(out, gates, ctx.buffer("gattn.act", (T, nh * V), ctx.dtype), nh, V, pad)
+        return ops.gemm(act, self.w_out, ctx.buffer("gattn.y", (T, self.hidden), torch.float32), scratch=ctx.scratch)
+
+    def forward(self, h, residual, ctx, site, norm=None):
+        return ops.residual_add(residual, self.output(h, ctx, site))
+
+
 register_part("mixer", "attention", PagedAttention)
+register_part("mixer", "normed_gated_attention", NormedGatedAttention)

@@ -1,6 +1,8 @@
 """Arrangement of parts in a layer.  PreNormBlock is the Llama arrangement
 (reference: runtime/model.py:106-119): x = x + mixer(norm1(x)); x = x + ffn(norm2(x)),
-the residual stream x kept in float."""
+the residual stream x kept in float.  SandwichBlock norms each sublayer's result as well
+and scales it: x = x + m norm1b(mixer(norm1(x))); x = x + m norm2b(ffn(norm2(x)))."""
+from ..kernels import ops
 from .base import Part, register_part
 
 
@@ -66,4 +68,87 @@ class PreNormBlock(Part):
         return self.ffn.forward(h, residual, ctx)
 
 
+class NormedMean:
+    """What a mixer made of two mixers side by side hands to the arrangement around it: half the sum of two results,
+    each RMS-normed over the width with a weight of its own (float [T, H] each).  The arrangement's kernel that adds
+    a sublayer's result to the residual stream makes the mean on the way (ops.post_norm_add)."""
+
+    def __init__(self, first, first_weight, second, second_weight, eps):
+        self.first, self.first_weight, self.second, self.second_weight, self.eps = first, first_weight, second, second_weight, eps
+
+
+def add_sublayer(residual, result, norm, mult, eps=None):
+    """residual += mult * norm(result) (norm None: mult * result); `result` float rows or a NormedMean."""
+    weight = None if norm is None else norm.weight
+    eps = norm.eps if norm is not None else eps
+    if isinstance(result, NormedMean):
+        if eps is not None and eps != result.eps:
+            raise ValueError("the norms inside a mean of two results and the norm around it must share their eps (one kernel)")
+        return ops.post_norm_add(residual, result.first, weight, result.eps, mult,
+                                 second=(result.second, result.first_weight, result.second_weight))
+    return ops.post_norm_add(residual, result, weight, 0.0 if eps is None else eps, mult)
+
+
+class SandwichBlock(Part):
+    """A norm before and after each sublayer, the normed result times `mult` added to the float residual stream.
+    Its mixer and feed-forward give their result without the residual sum (`output`); `ffn` None: a layer without
+    a feed-forward.  The norms after the sublayers are RMS norms (`weight`, `eps`); the sum, the norm and the scale
+    are one kernel."""
+
+    def __init__(self, mixer_norm, mixer, mixer_post, ffn_norm=None, ffn=None, ffn_post=None, mult=1.0):
+        if (ffn is None) != (ffn_norm is None) or (ffn is None) != (ffn_post is None):
+            raise ValueError("a feed-forward comes with the norms before and after it, or not at all")
+        for post in (mixer_post, ffn_post):
+            if post is not None and getattr(post, "fusable_as", None) != "rms":
+                raise ValueError("the norm after a sublayer must be an RMS norm (weight, eps)")
+        if not hasattr(mixer, "output") or (ffn is not None and not hasattr(ffn, "output")):
+            raise ValueError("the sublayers of this arrangement must give their result without the residual sum (output)")
+        self.mixer_norm, self.mixer, self.mixer_post = mixer_norm, mixer, mixer_post
+        self.ffn_norm, self.ffn, self.ffn_post = ffn_norm, ffn, ffn_post
+        self.mult = float(mult)
+
+    def parts(self):
+        return [p for p in (self.mixer_norm, self.mixer, self.mixer_post, self.ffn_norm, self.ffn, self.ffn_post) if p is not None]
+
+    def tensor_specs(self):
+        return [s for p in self.parts() for s in p.tensor_specs()]
+
+    def bind(self, tensors, dtype):
+        for p in self.parts():
+            p.bind(tensors, dtype)
+
+    def prepare(self, device, dtype):
+        for p in self.parts():
+            p.prepare(device, dtype)
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def cache_read(self):
+        return self.mixer.cache_read()
+
+    def state_need(self):
+        return self.mixer.state_need()
+
+    def kernel_units(self, dtype):
+        return [u for p in self.parts() if hasattr(p, "kernel_units") for u in p.kernel_units(dtype)]
+
+    def step_arrays(self):
+        return [a for p in self.parts() if hasattr(p, "step_arrays") for a in p.step_arrays()]
+
+    def first_norm(self):
+        return self.mixer_norm
+
+    def forward(self, residual, ctx, site):
+        ctx.next_norm = None          # (no product of this block is left to a later norm)
+        h = self.mixer_norm.forward(residual, ctx)
+        ctx.settle(residual)
+        add_sublayer(residual, self.mixer.output(h, ctx, site), self.mixer_post, self.mult)
+        if self.ffn is not None:
+            h = self.ffn_norm.forward(residual, ctx)
+            add_sublayer(residual, self.ffn.output(h, ctx), self.ffn_post, self.mult)
+        return residual
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "sandwich", SandwichBlock)

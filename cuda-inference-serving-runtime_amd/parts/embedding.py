@@ -11,15 +11,17 @@ from .base import Part, TensorSpec, matrix_operand
 
 
 class TokenEmbedding(Part):
-    def __init__(self, name, vocab, hidden):
+    def __init__(self, name, vocab, hidden, tensor=None):
+        """`tensor`: the table's full name where it is not `<name>.weight`."""
         self.name, self.vocab, self.hidden = name, vocab, hidden
+        self.tensor = tensor if tensor is not None else name + ".weight"
         self.weight = None
 
     def tensor_specs(self):
-        return [TensorSpec(self.name + ".weight", (self.vocab, self.hidden))]
+        return [TensorSpec(self.tensor, (self.vocab, self.hidden))]
 
     def bind(self, tensors, dtype):
-        self.weight = matrix_operand(tensors[self.name + ".weight"], dtype)
+        self.weight = matrix_operand(tensors[self.tensor], dtype)
 
     def forward(self, ctx):
         out = ctx.buffer("residual", (ctx.tokens.shape[0], self.hidden), torch.float32)
@@ -27,15 +29,16 @@ class TokenEmbedding(Part):
 
 
 class LMHead(Part):
-    def __init__(self, name, vocab, hidden, tied_to=None):
+    def __init__(self, name, vocab, hidden, tied_to=None, tensor=None):
         self.name, self.vocab, self.hidden, self.tied_to = name, vocab, hidden, tied_to
+        self.tensor = tensor if tensor is not None else name + ".weight"
         self.weight = None
 
     def tensor_specs(self):
-        return [] if self.tied_to is not None else [TensorSpec(self.name + ".weight", (self.vocab, self.hidden))]
+        return [] if self.tied_to is not None else [TensorSpec(self.tensor, (self.vocab, self.hidden))]
 
     def bind(self, tensors, dtype):
-        self.weight = self.tied_to.weight if self.tied_to is not None else matrix_operand(tensors[self.name + ".weight"], dtype)
+        self.weight = self.tied_to.weight if self.tied_to is not None else matrix_operand(tensors[self.tensor], dtype)
 
     def fuses_norm(self, norm, residual, rows):
         return getattr(norm, "fusable_as", None) == "rms" and ops.fused_norm_ok(residual, self.weight, rows.shape[0])

@@ -52,4 +52,39 @@ class GatedMLP(FeedForward):
         return ctx.add_product(act, self.w_down, residual)
 
 
+class ClampedGLU(FeedForward):
+    """y = (g sigmoid(slope g) (u + shift)) Wd^T with g = min(h Wg^T, limit), u = clamp(h Wu^T, -limit, limit).
+    Gate and up run as one product against [gate; up]; `names` = (gate, up, down), the tensors' names under `name`."""
+
+    def __init__(self, name, hidden, intermediate, limit, slope=1.702, shift=1.0, names=("gate", "up", "down")):
+        if not limit > 0:
+            raise ValueError("the clamp's limit must be positive")
+        self.name, self.hidden, self.intermediate = name, hidden, intermediate
+        self.limit, self.slope, self.shift, self.names = float(limit), float(slope), float(shift), tuple(names)
+        self.w_gate_up = self.w_down = None
+
+    def _tensor(self, which):
+        return f"{self.name}.{self.names[which]}"
+
+    def tensor_specs(self):
+        H, I = self.hidden, self.intermediate
+        return [TensorSpec(self._tensor(0), (I, H)), TensorSpec(self._tensor(1), (I, H)), TensorSpec(self._tensor(2), (H, I))]
+
+    def bind(self, tensors, dtype):
+        gate, up = (matrix_operand(tensors[self._tensor(i)], dtype) for i in (0, 1))
+        self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
+        self.w_down = matrix_operand(tensors[self._tensor(2)], dtype)
+
+    def output(self, h, ctx):
+        """The feed-forward's result, float [T, hidden], without the residual sum."""
+        T = h.shape[0]
+        gate_up = ops.gemm(h, self.w_gate_up, ctx.buffer("ffn.gate_up", (T, 2 * self.intermediate), ctx.dtype), scratch=ctx.scratch)
+        act = ops.glu_clamped(gate_up, ctx.buffer("ffn.act", (T, self.intermediate), ctx.dtype), self.limit, self.slope, self.shift)
+        return ops.gemm(act, self.w_down, ctx.buffer("ffn.out", (T, self.hidden), torch.float32), scratch=ctx.scratch)
+
+    def forward(self, h, residual, ctx, norm=None):
+        return ops.residual_add(residual, self.output(h, ctx))
+
+
 register_part("ffn", "gated_mlp", GatedMLP)
+register_part("ffn", "clamped_glu", ClampedGLU)

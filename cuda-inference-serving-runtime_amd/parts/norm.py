@@ -12,15 +12,17 @@ class RMSNorm(Part):
     fusable_as = "rms"
     adds_partials = True    # forward adds the partial sums of a product left unfinished before it (ctx.add_product)
 
-    def __init__(self, name, dim, eps):
+    def __init__(self, name, dim, eps, tensor=None):
+        """`tensor`: the weight's full name where it is not `<name>.weight`."""
         self.name, self.dim, self.eps = name, dim, float(eps)
+        self.tensor = tensor if tensor is not None else name + ".weight"
         self.weight = None
 
     def tensor_specs(self):
-        return [TensorSpec(self.name + ".weight", (self.dim,), init="one_plus_normal")]
+        return [TensorSpec(self.tensor, (self.dim,), init="one_plus_normal")]
 
     def bind(self, tensors, dtype):
-        self.weight = tensors[self.name + ".weight"].to(torch.float32).contiguous()  # exact widening
+        self.weight = tensors[self.tensor].to(torch.float32).contiguous()  # exact widening
 
     def forward(self, x, ctx, rows=None, tag="norm"):
         n_out = x.shape[0] if rows is None else rows.shape[0]

@@ -1,0 +1,202 @@
+"""Mixers that keep a state of fixed size per request instead of keys and values.
+
+Both are the same recurrence per head, S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t, run by one kernel
+(ops.linear_scan) over the rows of a step as they come (portions and single tokens of several requests), with
+the state in the cache manager's state slots, in float in every mode:
+
+  GatedLinearAttention   a_t a vector over the key channels, sigmoid(z_t)^(1/tau), z_t from a low-rank projection
+                         with a bias; q scaled by dim^(-1/2); each head's result RMS-normed over vdim with a weight
+                         shared by the heads, times silu of a gate projection, then the output projection.
+  StateSpaceDuality      (Mamba-2) a_t one number a head, exp(-exp(A_log) dt_t) with dt_t = softplus(dt + dt_bias);
+                         k = B_t, q = C_t (shared by the heads of a group), v = dt_t x_t; x, B and C come out of a short
+                         causal convolution with silu whose last inputs are part of the state; y = o + D x, times
+                         silu(z), RMS-normed in equal parts of the row, then the output projection.
+
+The projections and the convolution's inputs are products with float results; decays, step sizes, gates of the
+recurrence and the norms are float arithmetic; the operands of the output projections are the compute dtype.
+"""
+import torch
+
+from ..cache.pages import StateNeed
+from ..kernels import library, ops
+from ..weights.loader import AnySize
+from .base import Mixer, TensorSpec, matrix_operand, register_part
+
+
+def _float(t):
+    return t.to(torch.float32).contiguous()
+
+
+class GatedLinearAttention(Mixer):
+    NAMES = {"q": "q", "k": "k", "v": "v", "gate": "g", "o": "o", "norm": "norm", "down": "a1", "up": "a2", "bias": "a2.b"}
+
+    def __init__(self, name, hidden, heads, dim, vdim, tau, eps, rank=16, names=None):
+        """`rank`: the inner size of the decay's low-rank projection where no file says it (the files decide)."""
+        if not tau > 0:
+            raise ValueError("tau must be positive")
+        self.name, self.hidden, self.heads, self.dim, self.vdim = name, hidden, heads, dim, vdim
+        self.tau, self.eps, self.rank = float(tau), float(eps), int(rank)
+        self.names = {**self.NAMES, **(names or {})}
+
+    def _tensor(self, which):
+        return f"{self.name}.{self.names[which]}"
+
+    def kernel_units(self, dtype):
+        return [library.RECURRENCE]
+
+    def state_need(self):
+        return StateNeed((self.heads, self.dim, self.vdim), "float32")
+
+    def tensor_specs(self):
+        H, K, V = self.hidden, self.heads * self.dim, self.heads * self.vdim
+        return [TensorSpec(self._tensor("q"), (K, H)), TensorSpec(self._tensor("k"), (K, H)), TensorSpec(self._tensor("v"), (V, H)),
+                TensorSpec(self._tensor("gate"), (V, H)), TensorSpec(self._tensor("o"), (H, V)),
+                TensorSpec(self._tensor("norm"), (self.vdim,), init="one_plus_normal"),
+                TensorSpec(self._tensor("down"), (AnySize(self.rank), H)), TensorSpec(self._tensor("up"), (K, AnySize(self.rank))),
+                TensorSpec(self._tensor("bias"), (K,))]
+
+    def bind(self, tensors, dtype):
+        self.w_in = torch.cat([matrix_operand(tensors[self._tensor(p)], dtype) for p in ("q", "k", "v", "gate")], dim=0).contiguous()
+        self.w_down, self.w_up = matrix_operand(tensors[self._tensor("down")], dtype), matrix_operand(tensors[self._tensor("up")], dtype)
+        if self.w_down.shape[0] != self.w_up.shape[1]:
+            raise ValueError(f"{self.name}: the decay's projections disagree about their inner size "
+                             f"({self.w_down.shape[0]} and {self.w_up.shape[1]})")
+        self.w_out = matrix_operand(tensors[self._tensor("o")], dtype)
+        self.norm_weight, self.bias = _float(tensors[self._tensor("norm")]), _float(tensors[self._tensor("bias")])
+
+    def output(self, h, ctx, site):
+        T = h.shape[0]
+        K, V = self.heads * self.dim, self.heads * self.vdim
+        proj = ops.gemm(h, self.w_in, ctx.buffer("gla.proj", (T, 2 * K + 2 * V), torch.float32), scratch=ctx.scratch)
+        low = ops.gemm(h, self.w_down, ctx.buffer("gla.low", (T, self.w_down.shape[0]), ctx.dtype), scratch=ctx.scratch)
+        z = ops.gemm(low, self.w_up, ctx.buffer("gla.decay", (T, K), torch.float32), scratch=ctx.scratch)
+        decay = ops.decay_gate(z, self.bias, z, self.tau)          # (in place: an element is read and written by one thread)
+        state = ctx.cache.state_storage[site]
+        o = ctx.buffer("gla.o", (T, V), torch.float32)
+        ops.linear_scan(proj[:, :K], proj[:, K:2 * K], proj[:, 2 * K:2 * K + V], decay, o, state.view(state.shape[0], -1),
+                        ctx.seg_start, ctx.state_slots, self.heads, self.dim, self.vdim, q_scale=self.dim ** -0.5)
+        act = ops.group_norm_gate(o, proj[:, 2 * K + V:], self.norm_weight, ctx.buffer("gla.act", (T, V), ctx.dtype),
+                                  self.heads, self.eps, gate_first=False, shared_weight=True)
+        return ops.gemm(act, self.w_out, ctx.buffer("gla.y", (T, self.hidden), torch.float32), scratch=ctx.scratch)
+
+    def forward(self, h, residual, ctx, site, norm=None):
+        return ops.residual_add(residual, self.output(h, ctx, site))
+
+
+class StateSpaceDuality(Mixer):
+    NAMES = {"in": "in", "conv": "conv", "conv_bias": "conv.b", "dt_bias": "dt_bias", "a_log": "A_log", "skip": "D",
+             "norm": "norm", "o": "o"}
+    MAX_TAPS = 16
+
+    def __init__(self, name, hidden, heads, vdim, state, groups, taps, norm_groups, eps, names=None):
+        if heads % groups:
+            raise ValueError(f"{heads} heads do not divide into {groups} groups")
+        if (heads * vdim) % norm_groups:
+            raise ValueError(f"{heads} x {vdim} channels do not divide into {norm_groups} equal parts")
+        if not 1 <= taps <= self.MAX_TAPS:
+            raise ValueError(f"a convolution of {taps} taps: 1 to {self.MAX_TAPS}")
+        self.name, self.hidden, self.heads, self.vdim, self.state, self.groups = name, hidden, heads, vdim, state, groups
+        self.taps, self.norm_groups, self.eps = int(taps), int(norm_groups), float(eps)
+        self.inner = heads * vdim
+        self.channels = self.inner + 2 * groups * state          # what the convolution runs over: x, B, C
+        self.names = {**self.NAMES, **(names or {})}
+
+    def _tensor(self, which):
+        return f"{self.name}.{self.names[which]}"
+
+    def kernel_units(self, dtype):
+        return [library.RECURRENCE]
+
+    def state_need(self):
+        """One float row a request: the heads' states [heads, state, vdim], then the convolution's last taps - 1 inputs
+        [taps - 1, channels]."""
+        return StateNeed((self.heads * self.state * self.vdim + (self.taps - 1) * self.channels,), "float32")
+
+    def tensor_specs(self):
+        H, t = self.hidden, self._tensor
+        return [TensorSpec(t("in"), (2 * self.inner + 2 * self.groups * self.state + self.heads, H)),
+                TensorSpec(t("conv"), (self.channels, self.taps)), TensorSpec(t("conv_bias"), (self.channels,)),
+                TensorSpec(t("dt_bias"), (self.heads,)), TensorSpec(t("a_log"), (self.heads,)), TensorSpec(t("skip"), (self.heads,)),
+                TensorSpec(t("norm"), (self.inner,), init="one_plus_normal"), TensorSpec(t("o"), (H, self.inner))]
+
+    def bind(self, tensors, dtype):
+        t = self._tensor
+        self.w_in, self.w_out = matrix_operand(tensors[t("in")], dtype), matrix_operand(tensors[t("o")], dtype)
+        self.conv, self.conv_bias = _float(tensors[t("conv")]), _float(tensors[t("conv_bias")])
+        self.dt_bias, self.a_log, self.skip = _float(tensors[t("dt_bias")]), _float(tensors[t("a_log")]), _float(tensors[t("skip")])
+        self.norm_weight = _float(tensors[t("norm")])
+
+    def output(self, h, ctx, site):
+        T = h.shape[0]
+        inner, GN, ch, nh = self.inner, self.groups * self.state, self.channels, self.heads
+        proj = ops.gemm(h, self.w_in, ctx.buffer("ssd.proj", (T, 2 * inner + 2 * GN + nh), torch.float32), scratch=ctx.scratch)
+        state = ctx.cache.state_storage[site]
+        heads_state = nh * self.state * self.vdim
+        xbc = ctx.buffer("ssd.xbc", (T, ch), torch.float32)
+        step, decay = ctx.buffer("ssd.step", (T, nh), torch.float32), ctx.buffer("ssd.decay", (T, nh), torch.float32)
+        ops.conv_silu(proj[:, inner:inner + ch], self.conv, self.conv_bias, state[:, heads_state:], xbc, ctx.seg_of_row,
+                      ctx.seg_start, ctx.state_slots, gates=(proj[:, inner + ch:], self.dt_bias, self.a_log, step, decay))
+        y = ctx.buffer("ssd.o", (T, inner), torch.float32)
+        ops.linear_scan(xbc[:, inner + GN:], xbc[:, inner:inner + GN], xbc[:, :inner], decay, y, state, ctx.seg_start,
+                        ctx.state_slots, nh, self.state, self.vdim, share=nh // self.groups, step=step)
+        act = ops.group_norm_gate(y, proj[:, :inner], self.norm_weight, ctx.buffer("ssd.act", (T, inner), ctx.dtype),
+                                  self.norm_groups, self.eps, gate_first=True, skip=(self.skip, xbc[:, :inner]))
+        return ops.gemm(act, self.w_out, ctx.buffer("ssd.y", (T, self.hidden), torch.float32), scratch=ctx.scratch)
+
+    def forward(self, h, residual, ctx, site, norm=None):
+        return ops.residual_add(residual, self.output(h, ctx, site))
+
+
+class SideBySide(Mixer):
+    """Two mixers that read the same input; the result is half the sum of theirs, each RMS-normed over the model
+    width with a weight of its own (`<name>.<first_out>` / `<name>.<second_out>`).  At most one of the two keeps pages
+    and at most one a state: a site of the cache has one need of each kind."""
+
+    def __init__(self, name, hidden, first, second, eps, first_out="left.out", second_out="right.out"):
+        for kind in ("cache_need", "state_need"):
+            if getattr(first, kind)() is not None and getattr(second, kind)() is not None:
+                raise ValueError(f"both mixers of {name} declare a {kind}: a layer keeps one")
+        self.name, self.hidden, self.first, self.second, self.eps = name, hidden, first, second, float(eps)
+        self.out_names = (f"{name}.{first_out}", f"{name}.{second_out}")
+
+    def mixers(self):
+        return [self.first, self.second]
+
+    def kernel_units(self, dtype):
+        return [u for m in self.mixers() if hasattr(m, "kernel_units") for u in m.kernel_units(dtype)]
+
+    def step_arrays(self):
+        return [a for m in self.mixers() if hasattr(m, "step_arrays") for a in m.step_arrays()]
+
+    def cache_need(self):
+        return self.first.cache_need() or self.second.cache_need()
+
+    def state_need(self):
+        return self.first.state_need() or self.second.state_need()
+
+    def tensor_specs(self):
+        return ([s for m in self.mixers() for s in m.tensor_specs()]
+                + [TensorSpec(n, (self.hidden,), init="one_plus_normal") for n in self.out_names])
+
+    def bind(self, tensors, dtype):
+        for m in self.mixers():
+            m.bind(tensors, dtype)
+        self.out_weights = [_float(tensors[n]) for n in self.out_names]
+
+    def prepare(self, device, dtype):
+        for m in self.mixers():
+            m.prepare(device, dtype)
+
+    def output(self, h, ctx, site):
+        from .block import NormedMean
+        return NormedMean(self.first.output(h, ctx, site), self.out_weights[0], self.second.output(h, ctx, site),
+                          self.out_weights[1], self.eps)
+
+    def forward(self, h, residual, ctx, site, norm=None):
+        from .block import add_sublayer
+        return add_sublayer(residual, self.output(h, ctx, site), None, 1.0)
+
+
+register_part("mixer", "gated_linear_attention", GatedLinearAttention)
+register_part("mixer", "state_space_duality", StateSpaceDuality)
+register_part("mixer", "side_by_side", SideBySide)

@@ -1,3 +1,3 @@
 from .safetensors_io import SafetensorsFile, SafetensorsError, write_safetensors
-from .loader import TensorSpec, WeightError, open_folder, check_against, load_folder
+from .loader import TensorSpec, AnySize, WeightError, open_folder, check_against, load_folder
 from .random_init import random_tensors, write_model_folder

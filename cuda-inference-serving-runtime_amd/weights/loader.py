@@ -34,11 +34,28 @@ class WeightError(ValueError):
 
 
 @dataclass(frozen=True)
+class AnySize:
+    """A dimension that the file decides, not the configuration (the rank of a low-rank projection); `default` is
+    what the random-weights mode draws.  The part that owns the tensor checks at `bind` whatever must agree."""
+    default: int
+
+    def __repr__(self):
+        return "any"
+
+
+@dataclass(frozen=True)
 class TensorSpec:
     name: str
-    shape: Tuple[int, ...]
+    shape: Tuple[object, ...]   # sizes; an AnySize stands for a dimension that the file decides
     init: str = "normal"        # "normal": N(0, std); "one_plus_normal": 1 + N(0, std)  (random-weights mode)
     integer: bool = False       # an integer table (kept as int32)
+
+    def fits(self, shape):
+        return len(shape) == len(self.shape) and all(isinstance(e, AnySize) or e == g for e, g in zip(self.shape, shape))
+
+    def drawn_shape(self):
+        """The shape the random-weights mode gives the tensor."""
+        return tuple(e.default if isinstance(e, AnySize) else e for e in self.shape)
 
 
 def open_folder(folder):
@@ -70,7 +87,7 @@ def check_against(specs, index, ignored=(), strict=False):
     for name, spec in expected.items():
         if name in index:
             _, shape = index[name].info(name)
-            if tuple(shape) != tuple(spec.shape):
+            if not spec.fits(tuple(shape)):
                 wrong.append(f"{name}: file has {list(shape)}, model expects {list(spec.shape)}")
     if missing or wrong or (strict and unexpected):
         lines = ["checkpoint does not match the model:"]

@@ -25,7 +25,7 @@ def random_tensors(specs, seed, dtype=torch.bfloat16, std=STD):
     for spec in sorted(specs, key=lambda s: s.name):
         if spec.integer:
             raise ValueError(f"{spec.name}: integer tables have no random initialisation")
-        values = rng.standard_normal(size=spec.shape, dtype=np.float32) * np.float32(std)
+        values = rng.standard_normal(size=spec.drawn_shape(), dtype=np.float32) * np.float32(std)
         if spec.init == "one_plus_normal":
             values = values + np.float32(1.0)
         out[spec.name] = torch.from_numpy(values).to(dtype)
