@@ -42,8 +42,8 @@ class Trace:
     def lines(self):
         return [json.dumps(s) for s in self.steps]
 
-    def check(self, folder, out_dir, dtype, vocab, sequences):
-        """sequences: {id: full token list}.  Compares every written row."""
+    def check(self, folder, out_dir, dtype, vocab, sequences, plain=plain_logits):
+        """sequences: {id: full token list}.  Compares every written row with `plain(folder, tokens)` [T, vocab]."""
         per_request = {}
         for step, rows in self.expect.items():
             data = np.fromfile(out_dir / f"{step}.f32", dtype="<f4").reshape(len(rows), vocab)
@@ -52,7 +52,7 @@ class Trace:
         written = {int(p.stem) for p in out_dir.glob("*.f32")}
         assert written == set(self.expect), "a step without wanted rows wrote a file, or a wanted one is missing"
         for rid, items in per_request.items():
-            ref = plain_logits(folder, sequences[rid])
+            ref = plain(folder, sequences[rid])
             pos = [p for p, _ in items]
             assert_close(np.stack([r for _, r in items]), ref[pos], dtype, what=f"request {rid}")
         return per_request
