@@ -272,7 +272,7 @@ def main():
     ap.add_argument("--overlap", type=int, default=1, choices=[0, 1],
                     help="1: picked tokens stay on the device and a step is launched before the tokens of the one "
                          "before are read, as the scheduler's overlapped ticks do; 0: every step waits for its tokens")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serving"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "designs"],
                     help="decode: fixed batches after whole prompts, timed per step (the default; its line also holds longer "
                          "contexts, further layer sizes and one serving run); serving: only --requests requests with prompts of "
                          "128..--prompt tokens and --new-tokens each through the scheduler, at --model's sizes")
@@ -281,10 +281,15 @@ def main():
     ap.add_argument("--token-budget", type=int, default=2112, help="serving: rows a step (a whole prompt beside 64 decoded tokens)")
     ap.add_argument("--prefill-chunk", type=int, default=2048)
     ap.add_argument("--check", type=int, default=1, choices=[0, 1], help="compare the timed way of running with the plain one first")
+    ap.add_argument("--widths", default="1024,2048,4096", help="designs workload: model widths to time (comma separated)")
+    ap.add_argument("--design-layers", type=int, default=4, help="designs workload: layers of each model")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only; --gpus {args.gpus} is not run")
         return 2
+    if args.workload == "designs":
+        print(json.dumps(designs(args)))
+        return 0
 
     import torch
     from runtime.config import preset
@@ -379,6 +384,86 @@ def main():
         line["sizes"] = sizes
     print(json.dumps(line))
     return 0
+
+
+def design_configs(width, layers, context):
+    """A Llama and a Novosun configuration of the same width, depth, feed-forward size and vocabulary.  The Novosun
+    layers alternate: softmax attention (heads of 64 for keys, 128 for values, a quarter as many key/value heads) beside
+    a state-space layer (inner size twice the width in heads of 64, 128 states, a convolution of 4 taps), then gated
+    linear attention (key size half the width, value size the width, in heads of 128 x 256)."""
+    ff, vocab = 4 * width, 32768
+    llama = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "vocab_size": vocab, "hidden_size": width,
+             "intermediate_size": ff, "num_hidden_layers": layers, "num_attention_heads": width // 128,
+             "num_key_value_heads": max(1, width // 512), "head_dim": 128, "rms_norm_eps": 1e-5, "rope_theta": 10000.0,
+             "max_position_embeddings": context, "tie_word_embeddings": False}
+    mlp = {"kind": "dense", "ff": ff, "limit": 7.0}
+    side = {"type": "parallel", "mlp": mlp, "mixer": {
+        "left": {"heads": width // 128, "kv_heads": max(1, width // 512), "dim": 64, "vdim": 128, "scale": 0.125},
+        "right": {"heads": 2 * width // 64, "vdim": 64, "state": 128, "groups": 1, "conv": 4, "norm_groups": 1}}}
+    gla = {"type": "gla", "mlp": mlp, "mixer": {"heads": width // 256, "dim": 128, "vdim": 256, "tau": 16.0}}
+    novosun = {"architecture": "Novosun", "vocab": vocab, "width": width, "residual_mult": 0.5, "norm": {"eps": 1e-5},
+               "layers": [side if i % 2 == 0 else gla for i in range(layers)], "max_positions": context}
+    return {"llama": llama, "novosun": novosun}
+
+
+def designs(args):
+    """Prompt steps and decode steps of the Novosun design beside the Llama design at equal width, depth, feed-forward
+    size and vocabulary (random weights drawn on the device): tokens a second of a whole prompt of --prompt tokens and
+    of decode steps of 1, 8 and 64 requests after such prompts, through the step function with captured programs and
+    the greedy pick."""
+    import statistics
+    import numpy as np
+    import torch
+    from runtime.engine import ModelRunner, StepEntry, random_model
+    from runtime.sampling import Sampler
+    sampler = Sampler()
+    rng = np.random.default_rng(0)
+    batches = [1, 8, 64]
+    steps, warmup, prompt = min(args.steps, 48), min(args.warmup, 8), args.prompt
+    context = prompt + 3 * steps + warmup + 16
+    out = {}
+    for width in [int(w) for w in args.widths.split(",") if w]:
+        for design, raw in design_configs(width, args.design_layers, context).items():
+            torch.cuda.empty_cache()
+            model = random_model(raw, seed=0, dtype=args.dtype)
+            parameters = sum(int(np.prod(s.drawn_shape())) for s in model.tensor_specs())
+            runner = ModelRunner(model, n_pages=-(-max(batches) * context // args.page_size) + 8, page_size=args.page_size,
+                                 max_requests=max(batches), execution=args.execution)
+            vocab = model.vocab_size
+            prefill, result = [], {"parameters": parameters}
+            for batch in batches:
+                keys = [f"{batch}-{i}" for i in range(batch)]
+                last = []
+                for key in keys:
+                    runner.create(key)
+                    tokens = rng.integers(0, vocab, size=prompt, dtype=np.int32)
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    last.append(sampler.pick(runner.step([StepEntry(key, tokens, [prompt - 1])]), [(0.0, 0, 0)])[0])
+                    torch.cuda.synchronize()
+                    prefill.append(time.perf_counter() - t0)
+                params = [(0.0, 0, 0)] * batch
+                timings = []
+                for repeat in range(4):                      # the first repeat warms up (eager run, capture)
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    for _ in range(warmup if repeat == 0 else steps):
+                        last = sampler.pick(runner.step([StepEntry(k, [t], [0]) for k, t in zip(keys, last)]), params)
+                    torch.cuda.synchronize()
+                    if repeat:
+                        timings.append((time.perf_counter() - t0) / steps)
+                for key in keys:
+                    runner.release(key)
+                result[f"decode_b{batch}"] = {"tokens_per_s": round(batch / statistics.median(timings), 1),
+                                              "ms_per_step": round(statistics.median(timings) * 1e3, 4)}
+            pf = statistics.median(prefill[2:])
+            result["prefill"] = {"tokens": prompt, "ms": round(pf * 1e3, 3), "tokens_per_s": round(prompt / pf, 1)}
+            out.setdefault(str(width), {})[design] = result
+            del runner, model
+    return {"metric": f"prompt and decode tokens/s of the Novosun design beside Llama at equal width, {args.design_layers} layers",
+            "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "steps": steps,
+            "data": "synthetic (random weights N(0,0.02), uniform-random token ids)", "prompt_len": prompt,
+            "execution": args.execution, "widths": out}
 
 
 def serving(args, model, name, full_layers):

@@ -15,110 +15,39 @@
 // without rows (padding of a captured step) touches nothing.  All of it is float arithmetic on float data: what
 // enters a recurrence is 32-bit in every mode.
 #include "common.h"
+#include "recurrence_scan.inc"
 
 // ------------------------------------------------------------------------------------------------ linear scan
-struct ScanArgs {
-    const float* q; int ldq;          // q[t * ldq + (head / share) * R + r]
-    const float* k; int ldk;          // k[t * ldk + (head / share) * R + r]
-    const float* v; int ldv;          // v[t * ldv + head * C + c]
-    const float* a; int lda;          // VEC: a[t * lda + head * R + r]; else a[t * lda + head]
-    const float* vs; int ldvs;        // null, or the step size vs[t * ldvs + head] that multiplies v
-    float* out; int ldo;              // out[t * ldo + head * C + c]
-    float* state; long long slot_stride;   // state + slot * slot_stride + (head * R + r) * C + c
-    const int* seg_start; const int* state_slots;
-    int R, C, share;
-    float q_scale;
-};
-
-// A wave a (segment, head, tile of COLS columns).  Lane l owns column l % COLS and the rows l / COLS + (64 / COLS) i,
-// i < RPT, of the state, in registers, and walks the segment's rows in order; the products of a column meet over the
-// 64 / COLS lanes that share it.  Columns of S are independent, so a head is as many waves as it has tiles.
-template <int COLS, int RPT, bool VEC>
-__global__ void __launch_bounds__(64) linear_scan_kernel(ScanArgs p) {
-    constexpr int NG = WAVE / COLS;
-    const int seg = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
-    const int t0 = p.seg_start[seg], t1 = p.seg_start[seg + 1];
-    if (t1 <= t0) return;
-    const int c = blockIdx.z * COLS + lane % COLS, rg = lane / COLS;
-    const bool col_ok = c < p.C;
-    const int cc = col_ok ? c : p.C - 1;
-    const int R = p.R, C = p.C;
-    float* state = p.state + (long long)p.state_slots[seg] * p.slot_stride + (size_t)head * R * C;
-    const float* qh = p.q + (size_t)(head / p.share) * R;
-    const float* kh = p.k + (size_t)(head / p.share) * R;
-    const float* ah = p.a + (VEC ? (size_t)head * R : (size_t)head);
-    const float* vh = p.v + (size_t)head * C + cc;
-    float S[RPT];
-    int rows[RPT];
-    bool ok[RPT];
-#pragma unroll
-    for (int i = 0; i < RPT; ++i) {
-        const int r = rg + NG * i;
-        ok[i] = r < R;
-        rows[i] = ok[i] ? r : R - 1;
-        S[i] = ok[i] ? state[(size_t)rows[i] * C + cc] : 0.f;
-    }
-    for (int t = t0; t < t1; ++t) {
-        float v = vh[(size_t)t * p.ldv];
-        if (p.vs) v *= p.vs[(size_t)t * p.ldvs + head];
-        const float a1 = VEC ? 0.f : ah[(size_t)t * p.lda];
-        const float* qt = qh + (size_t)t * p.ldq;
-        const float* kt = kh + (size_t)t * p.ldk;
-        const float* at = ah + (size_t)t * p.lda;
-        float acc = 0.f;
-#pragma unroll
-        for (int i = 0; i < RPT; ++i) {
-            const float kk = ok[i] ? kt[rows[i]] : 0.f;      // (a row past R stays zero and adds nothing)
-            const float aa = VEC ? at[rows[i]] : a1;
-            S[i] = aa * S[i] + kk * v;
-            acc += S[i] * qt[rows[i]];
-        }
-#pragma unroll
-        for (int off = COLS; off < WAVE; off <<= 1) acc += __shfl_xor(acc, off, WAVE);
-        if (rg == 0 && col_ok) p.out[(size_t)t * p.ldo + (size_t)head * C + c] = acc * p.q_scale;
-    }
-    if (col_ok) {
-#pragma unroll
-        for (int i = 0; i < RPT; ++i)
-            if (ok[i]) state[(size_t)rows[i] * C + c] = S[i];
-    }
+// (the kernel: recurrence_scan.inc; one source file a tile width)
+// Floats of `carry` and of `carry_decay` that a launch over `rows` rows in pieces of `piece` rows needs.
+extern "C" long long cisr_linear_scan_carry(int rows, int piece, int heads, int R, int C, int vec, long long* decay_floats) {
+    const long long pieces = piece > 0 ? (rows + piece - 1) / piece : 0;     // (the segments' pieces but their last are at most rows / piece)
+    if (decay_floats) *decay_floats = pieces * heads * (vec ? R : 1);
+    return pieces * heads * R * C;
 }
 
-template <int COLS, int RPT>
-static int launch_scan(const ScanArgs& p, int segments, int heads, bool vec, hipStream_t stream) {
-    const dim3 grid(segments, heads, (p.C + COLS - 1) / COLS);
-    if (vec) linear_scan_kernel<COLS, RPT, true><<<grid, 64, 0, stream>>>(p);
-    else linear_scan_kernel<COLS, RPT, false><<<grid, 64, 0, stream>>>(p);
-    return CISR_LAUNCH_CHECK();
-}
+int cisr_scan_launch_c4(const ScanArgs& p, int segments, bool vec, hipStream_t stream);
+int cisr_scan_launch_c8(const ScanArgs& p, int segments, bool vec, hipStream_t stream);
+int cisr_scan_launch_c16(const ScanArgs& p, int segments, bool vec, hipStream_t stream);
 
-// cols: 4, 8 or 16 columns a wave (the caller's rule: fewer columns are more waves for the same head).
+// cols: 4, 8 or 16 columns a wave (the caller's rule: fewer columns are more waves for the same head).  piece > 0:
+// segments longer than `piece` rows are walked in pieces of that many rows side by side (three launches; `rows` is the
+// number of rows of the step, carry / carry_decay as cisr_linear_scan_carry says); piece 0: a wave walks a whole segment.
 extern "C" int cisr_linear_scan(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv,
                                 const float* a, int lda, int vec, const float* vs, int ldvs, float* out, int ldo,
                                 float* state, long long slot_stride, const int* seg_start, const int* state_slots,
                                 int segments, int heads, int R, int C, int share, float q_scale, int cols,
-                                hipStream_t stream) {
+                                int rows, int piece, float* carry, float* carry_decay, hipStream_t stream) {
     if (segments <= 0 || heads <= 0) return 0;
-    if (R <= 0 || C <= 0 || share <= 0 || heads % share || heads > 65535 || (cols != 4 && cols != 8 && cols != 16))
+    if (R <= 0 || C <= 0 || share <= 0 || heads % share || heads > 65535 || (cols != 4 && cols != 8 && cols != 16) ||
+        piece < 0 || (piece > 0 && (!carry || !carry_decay || rows <= 0)))
         return (int)hipErrorInvalidValue;
-    ScanArgs p{q, ldq, k, ldk, v, ldv, a, lda, vs, ldvs, out, ldo, state, slot_stride, seg_start, state_slots, R, C, share, q_scale};
-    const int per = (R + (WAVE / cols) - 1) / (WAVE / cols);    // rows a lane
-    if ((C + cols - 1) / cols > 65535) return (int)hipErrorInvalidValue;
-#define SCAN_CASE(COLS) \
-    if (cols == COLS) { \
-        if (per <= 2) return launch_scan<COLS, 2>(p, segments, heads, vec, stream); \
-        if (per <= 4) return launch_scan<COLS, 4>(p, segments, heads, vec, stream); \
-        if (per <= 8) return launch_scan<COLS, 8>(p, segments, heads, vec, stream); \
-        if (per <= 16) return launch_scan<COLS, 16>(p, segments, heads, vec, stream); \
-        if (per <= 32) return launch_scan<COLS, 32>(p, segments, heads, vec, stream); \
-        if (per <= 64) return launch_scan<COLS, 64>(p, segments, heads, vec, stream); \
-        return (int)hipErrorInvalidValue; \
-    }
-    SCAN_CASE(4)
-    SCAN_CASE(8)
-    SCAN_CASE(16)
-#undef SCAN_CASE
-    return (int)hipErrorInvalidValue;
+    ScanArgs p{q, ldq, k, ldk, v, ldv, a, lda, vs, ldvs, out, ldo, state, slot_stride, seg_start, state_slots, R, C, share, heads,
+               q_scale, piece, piece > 0 ? (rows + piece - 1) / piece : 1, 0, carry, carry_decay};
+    if ((C + cols - 1) / cols > 65535 || R > 256) return (int)hipErrorInvalidValue;
+    if (cols == 4) return cisr_scan_launch_c4(p, segments, vec, stream);
+    if (cols == 8) return cisr_scan_launch_c8(p, segments, vec, stream);
+    return cisr_scan_launch_c16(p, segments, vec, stream);
 }
 
 // ------------------------------------------------------------------------------------------------ short conv
@@ -222,24 +151,26 @@ extern "C" int cisr_decay_gate(const float* z, int ld, const float* bias, float*
 //   u = y[t, i] + (skip ? skip[i / skip_span] * x[t * ldx + i] : 0)
 //   GATE_FIRST:  u *= silu(gate[t * ldg + i]);  out = u / rms(part) * w[shared ? d : i]
 //   else:        out = u / rms(part) * w[shared ? d : i] * silu(gate[t * ldg + i])
-// A wave a (row, part); the part is read twice.
-template <typename T, bool GATE_FIRST>
-__global__ void __launch_bounds__(64)
+// A block of NT threads a (row, part): a wave for parts of up to 256 elements, four waves for longer ones; the part is
+// read twice.
+template <typename T, bool GATE_FIRST, int NT>
+__global__ void __launch_bounds__(NT)
 group_norm_gate_kernel(const float* __restrict__ y, const float* __restrict__ gate, int ldg, const float* __restrict__ w,
                        int shared, const float* __restrict__ skip, int skip_span, const float* __restrict__ x, int ldx,
                        T* __restrict__ out, int size, float eps) {
+    __shared__ float red[NT / WAVE];
     const int t = blockIdx.x, g = blockIdx.y, groups = gridDim.y, lane = threadIdx.x;
     const size_t base = (size_t)t * groups * size + (size_t)g * size;
     const int col0 = g * size;
     float ss = 0.f;
-    for (int d = lane; d < size; d += WAVE) {
+    for (int d = lane; d < size; d += NT) {
         float u = y[base + d];
         if (skip) u += skip[(col0 + d) / skip_span] * x[(size_t)t * ldx + col0 + d];
         if (GATE_FIRST) { const float z = gate[(size_t)t * ldg + col0 + d]; u *= z / (1.0f + expf(-z)); }
         ss += u * u;
     }
-    const float scale = 1.0f / sqrtf(wave_sum(ss) / (float)size + eps);
-    for (int d = lane; d < size; d += WAVE) {
+    const float scale = 1.0f / sqrtf((NT == WAVE ? wave_sum(ss) : block_sum<NT>(ss, red)) / (float)size + eps);
+    for (int d = lane; d < size; d += NT) {
         float u = y[base + d];
         if (skip) u += skip[(col0 + d) / skip_span] * x[(size_t)t * ldx + col0 + d];
         const float z = gate[(size_t)t * ldg + col0 + d];
@@ -257,7 +188,10 @@ extern "C" int cisr_group_norm_gate(const float* y, const float* gate, int ldg, 
     if (rows <= 0) return 0;
     if (groups <= 0 || groups > 65535 || size <= 0 || (skip && (skip_span <= 0 || !x))) return (int)hipErrorInvalidValue;
     const dim3 grid(rows, groups);
-#define GNG(T, GF) group_norm_gate_kernel<T, GF><<<grid, 64, 0, stream>>>(y, gate, ldg, w, shared, skip, skip_span, x, ldx, (T*)out, size, eps)
+#define GNG(T, GF) do { \
+        if (size <= 256) group_norm_gate_kernel<T, GF, 64><<<grid, 64, 0, stream>>>(y, gate, ldg, w, shared, skip, skip_span, x, ldx, (T*)out, size, eps); \
+        else group_norm_gate_kernel<T, GF, 256><<<grid, 256, 0, stream>>>(y, gate, ldg, w, shared, skip, skip_span, x, ldx, (T*)out, size, eps); \
+    } while (0)
     if (dtype == DT_F32) { if (gate_first) GNG(float, true); else GNG(float, false); }
     else { if (gate_first) GNG(bf16_t, true); else GNG(bf16_t, false); }
 #undef GNG

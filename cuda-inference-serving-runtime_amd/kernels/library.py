@@ -37,7 +37,7 @@ _libs = {}
 CORE = "kernels"                                   # everything but the matrix-core attention and the measurement kernels
 MEASURE = "measure"                                # kernels that only measure the machine; the engine never loads them
 RECURRENCE = "recurrence"                          # mixers with a state per request: scans, short convolutions, their gates
-OWN_UNITS = (MEASURE, RECURRENCE)                  # units of one source file of the same name
+OWN_UNITS = (MEASURE, RECURRENCE)                  # units of the source files whose names start with the unit's
 ATTENTION_PADS = (32, 64, 96, 128, 160, 192, 224, 256)
 
 
@@ -61,9 +61,9 @@ def units():
 
 def sources(unit=CORE):
     if unit == CORE:
-        return sorted(p for p in CSRC.glob("*.hip") if not p.name.startswith("attention_mfma_d") and p.stem not in OWN_UNITS)
+        return sorted(p for p in CSRC.glob("*.hip") if not p.name.startswith("attention_mfma_d") and not p.stem.startswith(OWN_UNITS))
     if unit in OWN_UNITS:
-        return [CSRC / f"{unit}.hip"]
+        return sorted(CSRC.glob(f"{unit}*.hip"))
     path = CSRC / f"attention_mfma_{unit[len('attn_'):]}.hip"
     if not path.exists():
         raise KernelLibraryError(f"no source for kernel unit {unit}")

@@ -899,7 +899,7 @@ def _rec():
         h = library.load(library.RECURRENCE)
         p, i, f, ll = C.c_void_p, C.c_int, C.c_float, C.c_longlong
         sig = {
-            "cisr_linear_scan": [p, i, p, i, p, i, p, i, i, p, i, p, i, p, ll, p, p, i, i, i, i, i, f, i, p],
+            "cisr_linear_scan": [p, i, p, i, p, i, p, i, i, p, i, p, i, p, ll, p, p, i, i, i, i, i, f, i, i, i, p, p, p],
             "cisr_conv_silu": [p, i, i, p, p, p, ll, p, p, p, p, i, i, i, i, i, i, p, p, p, p, p],
             "cisr_decay_gate": [p, i, p, p, i, i, f, p],
             "cisr_group_norm_gate": [p, p, i, p, i, p, i, p, i, p, i, i, i, f, i, i, p],
@@ -908,6 +908,8 @@ def _rec():
             fn = getattr(h, name)
             fn.argtypes = args
             fn.restype = C.c_int
+        h.cisr_linear_scan_carry.argtypes = [i, i, i, i, i, i, C.POINTER(ll)]
+        h.cisr_linear_scan_carry.restype = ll
         _recurrence = h
     return _recurrence
 
@@ -921,26 +923,45 @@ def _rows_of(t, name, cols=None):
     return t.data_ptr(), t.stride(0)
 
 
-def scan_columns(segments, heads, cols):
+def scan_piece(rows, decode_only):
+    """Rows of a piece where the linear scan walks long segments in pieces side by side (0: a wave walks a whole
+    segment).  A step of single tokens has nothing to cut; a portion is cut so that its pieces fill the GPU, at the
+    price of walking every piece but the last twice (once for its end state, once for its results)."""
+    if decode_only or rows < 128:
+        return 0
+    return 128 if rows >= 1024 else 64
+
+
+def scan_columns(runs, heads, cols):
     """Columns of the state that one wave of the linear scan owns (16, 8 or 4): fewer columns make more waves of the
-    same head, until the launch has about two waves for every SIMD of the GPU."""
+    same head, until the launch has about two waves for every SIMD of the GPU.  `runs`: segments, or pieces of them."""
     for width in (16, 8, 4):
-        if segments * heads * -(-cols // width) >= 2048 or width == 4:
+        if runs * heads * -(-cols // width) >= 2048 or width == 4:
             return width
 
 
+def scan_carry(rows, piece, heads, rows_of_state, cols_of_state, vector):
+    """(floats of carry, floats of carry_decay) that linear_scan needs for a step of `rows` rows cut into pieces."""
+    decay = C.c_longlong(0)
+    n = _rec().cisr_linear_scan_carry(int(rows), int(piece), int(heads), int(rows_of_state), int(cols_of_state), int(vector), C.byref(decay))
+    return int(n), int(decay.value)
+
+
 def linear_scan(q, k, v, decay, out, state, seg_start, state_slots, heads, rows_of_state, cols_of_state, share=1,
-                step=None, q_scale=1.0, columns=None):
+                step=None, q_scale=1.0, columns=None, piece=0, carry=None):
     """Per segment and head: S_t = diag(a_t) S_(t-1) + k_t (v_t step_t)^T, o_t = q_scale S_t^T q_t over the segment's
     rows in order, S [rows_of_state, cols_of_state] read from and written back to the segment's state slot.
     q, k float views [T, heads / share * R]; v, out [T, heads * C]; decay [T, heads * R] (a vector a head) or
     [T, heads] (a number a head); step None or [T, heads]; state float [slots, >= heads * R * C] (a view whose rows
-    start with the state); seg_start int32 [S + 1]; state_slots int32 [S]."""
+    start with the state); seg_start int32 [S + 1]; state_slots int32 [S].
+    `piece` > 0: segments longer than that many rows are walked in pieces side by side (three launches: the pieces'
+    end states from zero, the states at their starts in order, the results), with `carry` = (float buffer, float
+    buffer) of at least scan_carry(...) elements."""
     R, Cc = int(rows_of_state), int(cols_of_state)
     T = v.shape[0]
     segments = state_slots.shape[0]
-    if heads % share or R > 64 * 16:
-        raise KernelError("linear_scan: heads must divide into their groups and a state has at most 1024 rows")
+    if heads % share or R > 256:
+        raise KernelError("linear_scan: heads must divide into their groups and a state has at most 256 rows")
     qp, ldq = _rows_of(q, "q", heads // share * R)
     kp, ldk = _rows_of(k, "k", heads // share * R)
     vp, ldv = _rows_of(v, "v", heads * Cc)
@@ -954,13 +975,19 @@ def linear_scan(q, k, v, decay, out, state, seg_start, state_slots, heads, rows_
         raise KernelError("linear_scan: operands differ in rows")
     if state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < heads * R * Cc or not state.is_cuda:
         raise KernelError("linear_scan: the state must be float [slots, >= heads * R * C]")
-    cols = int(columns or scan_columns(segments, heads, Cc))
+    cp = dp = None
+    if piece:
+        need = scan_carry(T, piece, heads, R, Cc, vec)
+        if carry is None or carry[0].numel() < need[0] or carry[1].numel() < need[1]:
+            raise KernelError("linear_scan: pieces need the carry buffers that scan_carry sizes")
+        cp, dp = _dev(carry[0], "carry", torch.float32), _dev(carry[1], "carry_decay", torch.float32)
+    cols = int(columns or scan_columns(-(-T // piece) if piece else segments, heads, Cc))
     while -(-R // (64 // cols)) > 64:
         cols *= 2          # (a lane holds at most 64 rows of its column)
     _check(_rec().cisr_linear_scan(qp, ldq, kp, ldk, vp, ldv, ap, lda, int(vec), sp, lds, op, ldo, state.data_ptr(),
                                    state.stride(0), _dev(seg_start, "seg_start", torch.int32, (segments + 1,)),
                                    _dev(state_slots, "state_slots", torch.int32, (segments,)), segments, heads, R, Cc,
-                                   int(share), float(q_scale), cols, _stream()), "linear_scan")
+                                   int(share), float(q_scale), cols, T, int(piece), cp, dp, _stream()), "linear_scan")
     return out
 
 

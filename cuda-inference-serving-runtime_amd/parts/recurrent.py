@@ -27,6 +27,17 @@ def _float(t):
     return t.to(torch.float32).contiguous()
 
 
+def _scan(ctx, tag, q, k, v, decay, out, state, heads, rows, cols, **kw):
+    """ops.linear_scan over the step's segments; the segments of a step with long portions are walked in pieces."""
+    T = v.shape[0]
+    piece = ops.scan_piece(T, ctx.decode_only)
+    carry = None
+    if piece:
+        n, n_decay = ops.scan_carry(T, piece, heads, rows, cols, decay.shape[1] != heads)
+        carry = (ctx.buffer(tag + ".carry", (n,), torch.float32), ctx.buffer(tag + ".carry_decay", (n_decay,), torch.float32))
+    return ops.linear_scan(q, k, v, decay, out, state, ctx.seg_start, ctx.state_slots, heads, rows, cols, piece=piece, carry=carry, **kw)
+
+
 class GatedLinearAttention(Mixer):
     NAMES = {"q": "q", "k": "k", "v": "v", "gate": "g", "o": "o", "norm": "norm", "down": "a1", "up": "a2", "bias": "a2.b"}
 
@@ -73,8 +84,8 @@ class GatedLinearAttention(Mixer):
         decay = ops.decay_gate(z, self.bias, z, self.tau)          # (in place: an element is read and written by one thread)
         state = ctx.cache.state_storage[site]
         o = ctx.buffer("gla.o", (T, V), torch.float32)
-        ops.linear_scan(proj[:, :K], proj[:, K:2 * K], proj[:, 2 * K:2 * K + V], decay, o, state.view(state.shape[0], -1),
-                        ctx.seg_start, ctx.state_slots, self.heads, self.dim, self.vdim, q_scale=self.dim ** -0.5)
+        _scan(ctx, "gla", proj[:, :K], proj[:, K:2 * K], proj[:, 2 * K:2 * K + V], decay, o, state.view(state.shape[0], -1),
+              self.heads, self.dim, self.vdim, q_scale=self.dim ** -0.5)
         act = ops.group_norm_gate(o, proj[:, 2 * K + V:], self.norm_weight, ctx.buffer("gla.act", (T, V), ctx.dtype),
                                   self.heads, self.eps, gate_first=False, shared_weight=True)
         return ops.gemm(act, self.w_out, ctx.buffer("gla.y", (T, self.hidden), torch.float32), scratch=ctx.scratch)
@@ -137,8 +148,8 @@ class StateSpaceDuality(Mixer):
         ops.conv_silu(proj[:, inner:inner + ch], self.conv, self.conv_bias, state[:, heads_state:], xbc, ctx.seg_of_row,
                       ctx.seg_start, ctx.state_slots, gates=(proj[:, inner + ch:], self.dt_bias, self.a_log, step, decay))
         y = ctx.buffer("ssd.o", (T, inner), torch.float32)
-        ops.linear_scan(xbc[:, inner + GN:], xbc[:, inner:inner + GN], xbc[:, :inner], decay, y, state, ctx.seg_start,
-                        ctx.state_slots, nh, self.state, self.vdim, share=nh // self.groups, step=step)
+        _scan(ctx, "ssd", xbc[:, inner + GN:], xbc[:, inner:inner + GN], xbc[:, :inner], decay, y, state,
+              nh, self.state, self.vdim, share=nh // self.groups, step=step)
         act = ops.group_norm_gate(y, proj[:, :inner], self.norm_weight, ctx.buffer("ssd.act", (T, inner), ctx.dtype),
                                   self.norm_groups, self.eps, gate_first=True, skip=(self.skip, xbc[:, :inner]))
         return ops.gemm(act, self.w_out, ctx.buffer("ssd.y", (T, self.hidden), torch.float32), scratch=ctx.scratch)

@@ -80,6 +80,50 @@ def test_linear_scan_over_segments_with_states_carried_and_slots_used_again(head
     assert float(state[1, 0]) == 7.0 and float(state[0, -1]) == 7.0, "a slot or a tail that no segment named was written"
 
 
+@pytest.mark.parametrize("heads, share, R, C, vector, piece", [(2, 1, 24, 20, True, 64), (4, 2, 16, 8, False, 64), (1, 1, 130, 33, True, 128)])
+def test_linear_scan_in_pieces_side_by_side_equals_the_scan_in_order(heads, share, R, C, vector, piece):
+    """Long segments are cut into pieces that waves of their own walk (end states from zero, the states at the pieces'
+    starts in order, then the results): segments of several pieces, of exactly one and two pieces, of one row and of
+    one row more than a piece, starting from states that an earlier launch left, beside each other in one launch."""
+    from runtime.kernels import ops
+    rng = np.random.default_rng(R + C)
+    lengths = {"a": 4 * piece + 37, "b": 1, "c": 2 * piece, "d": piece + 1, "e": piece}
+    groups = heads // share
+    data, want = {}, {}
+    for key, n in lengths.items():
+        n2 = n + 12
+        d = data[key] = dict(q=rng.standard_normal((n2, groups, R)), k=rng.standard_normal((n2, groups, R)), v=rng.standard_normal((n2, heads, C)),
+                             a=rng.uniform(0.8, 1.0, (n2, heads, R if vector else 1)))
+        want[key] = np.stack([P.decayed_outer_scan(d["q"][:, h // share], d["k"][:, h // share], d["v"][:, h],
+                                                   np.broadcast_to(d["a"][:, h], (n2, R))) for h in range(heads)], axis=1)
+    state = torch.zeros((5, heads * R * C), device=DEV)
+    slots = {"a": 3, "b": 0, "c": 4, "d": 1, "e": 2}
+
+    def launch(spans, piece):
+        keys = list(spans)
+        rows = {name: np.concatenate([data[k][name][lo:hi].reshape(hi - lo, -1) for k, (lo, hi) in spans.items()]) for name in "qkva"}
+        starts = np.concatenate(([0], np.cumsum([hi - lo for lo, hi in spans.values()])))
+        T = len(rows["v"])
+        out = torch.zeros(rows["v"].shape, device=DEV)
+        carry = None
+        if piece:
+            n, n_decay = ops.scan_carry(T, piece, heads, R, C, vector)
+            carry = (torch.full((n,), 5.0, device=DEV), torch.full((n_decay,), 5.0, device=DEV))
+        ops.linear_scan(dev(rows["q"]), dev(rows["k"]), dev(rows["v"]), dev(rows["a"]), out, state, ints(starts), ints([slots[k] for k in keys]),
+                        heads, R, C, share=share, piece=piece, carry=carry)
+        return dict(zip(keys, np.split(out.cpu().numpy().reshape(-1, heads, C), starts[1:-1])))
+
+    first = launch({"a": (0, 9), "c": (0, 3), "e": (0, 2)}, 0)                       # some start from a state that is not zero
+    got = launch({k: ({"a": 9, "c": 3, "e": 2}.get(k, 0), n + {"a": 9, "c": 3, "e": 2}.get(k, 0)) for k, n in lengths.items()}, piece)
+    for k, n in lengths.items():
+        lo = {"a": 9, "c": 3, "e": 2}.get(k, 0)
+        close(got[k], want[k][lo:lo + n], 5e-5)
+    after = launch({k: (n + {"a": 9, "c": 3, "e": 2}.get(k, 0), n + {"a": 9, "c": 3, "e": 2}.get(k, 0) + 1) for k, n in lengths.items() if k != "b"}, 0)
+    for k in after:                                                                      # the states the pieces left
+        at = lengths[k] + {"a": 9, "c": 3, "e": 2}.get(k, 0)
+        close(after[k], want[k][at:at + 1], 5e-5)
+
+
 @pytest.mark.parametrize("channels, taps, heads", [(10, 4, 3), (7, 2, 1), (300, 3, 2), (5, 1, 2), (6, 16, 0)])
 def test_short_convolution_carries_its_last_inputs_across_portions_of_any_size(channels, taps, heads):
     from runtime.kernels import ops
