@@ -1,6 +1,7 @@
 // Row-wise kernels of layers that norm a sublayer's output before the residual sum, of feed-forwards with a
 // clamped gate, and of attention that norms its queries and keys per head and gates its heads:
-//   x += mult * rmsnorm(y) * w                      (also with y = (rmsnorm(a) wa + rmsnorm(b) wb) / 2 made on the way)
+//   x += mult * rmsnorm(y) * w                      (also with y = (rmsnorm(a) wa + rmsnorm(b) wb) / 2 made on the way,
+//                                                    and with the next norm of x made on the way)
 //   act = g sigmoid(slope g) (u + shift), g = min(gate, limit), u = clamp(up, -limit, limit)
 //   q, k normed per head, q into a buffer of padded heads, k and v into the pages of the cache
 //   out[t, h, :] = attn[t, h, :vdim] * sigmoid(gate[t, h])
@@ -9,13 +10,15 @@
 
 // ------------------------------------------------- norm of a sublayer's output, scaled, into the residual stream
 // One block a row.  TWO: the row is half the sum of two rows, each normed over the width with a weight of its own.
-// A row is read three times (its squares, the squares of what is normed, the sum): the second and third from cache.
-template <bool TWO>
+// With next_w the norm that reads the residual stream next is made on the way: next_out = rmsnorm(x) * next_w.
+// KEEP: the row waits in LDS between the passes (rows of up to 16,384 floats); else it is read again.
+template <bool TWO, bool KEEP, typename T>
 __global__ void __launch_bounds__(256)
 post_norm_add_kernel(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ wa,
                      const float* __restrict__ b, const float* __restrict__ wb, const float* __restrict__ w,
-                     int dim, float eps, float mult) {
+                     int dim, float eps, float mult, const float* __restrict__ next_w, float next_eps, T* __restrict__ next_out) {
     __shared__ float red[4];
+    extern __shared__ float kept[];
     const size_t row = blockIdx.x;
     const float* ar = a + row * dim;
     const float* br = TWO ? b + row * dim : nullptr;
@@ -24,6 +27,7 @@ post_norm_add_kernel(float* __restrict__ x, const float* __restrict__ a, const f
         const float u = ar[d];
         sa += u * u;
         if (TWO) { const float v = br[d]; sb += v * v; }
+        else if (KEEP) kept[d] = u;
     }
     float ra = 1.f, rb = 0.f;
     if (TWO) {
@@ -32,24 +36,48 @@ post_norm_add_kernel(float* __restrict__ x, const float* __restrict__ a, const f
         sa = 0.f;
         for (int d = threadIdx.x; d < dim; d += 256) {
             const float y = ar[d] * ra * wa[d] + br[d] * rb * wb[d];
+            if (KEEP) kept[d] = y;
             sa += y * y;
         }
     }
     // (w null: the row is added as it is, times mult)
     const float scale = w ? mult / sqrtf(block_sum<256>(sa, red) / (float)dim + eps) : mult;
     float* xr = x + row * dim;
-    for (int d = threadIdx.x; d < dim; d += 256) {
-        const float y = TWO ? ar[d] * ra * wa[d] + br[d] * rb * wb[d] : ar[d];
-        xr[d] += y * scale * (w ? w[d] : 1.0f);
+    float sn = 0.f;
+    for (int d = threadIdx.x; d < dim; d += 256) {         // (a thread reads back only what it wrote itself)
+        const float y = KEEP ? kept[d] : TWO ? ar[d] * ra * wa[d] + br[d] * rb * wb[d] : ar[d];
+        const float xn = xr[d] + y * scale * (w ? w[d] : 1.0f);
+        xr[d] = xn;
+        if (KEEP) kept[d] = xn;
+        sn += xn * xn;
     }
+    if (next_w == nullptr) return;
+    const float rs = 1.0f / sqrtf(block_sum<256>(sn, red) / (float)dim + next_eps);
+    T* out = next_out + row * dim;
+    for (int d = threadIdx.x; d < dim; d += 256) store_f32(out + d, (KEEP ? kept[d] : xr[d]) * rs * next_w[d]);
+}
+
+template <bool TWO, typename T>
+static void launch_post_norm_add(float* x, const float* a, const float* wa, const float* b, const float* wb, const float* w,
+                                 int rows, int dim, float eps, float mult, const float* next_w, float next_eps, T* next_out,
+                                 hipStream_t stream) {
+    if (dim <= 16384) post_norm_add_kernel<TWO, true, T><<<rows, 256, (size_t)dim * sizeof(float), stream>>>(x, a, wa, b, wb, w, dim, eps, mult, next_w, next_eps, next_out);
+    else post_norm_add_kernel<TWO, false, T><<<rows, 256, 0, stream>>>(x, a, wa, b, wb, w, dim, eps, mult, next_w, next_eps, next_out);
 }
 
 extern "C" int cisr_post_norm_add(float* x, const float* a, const float* wa, const float* b, const float* wb,
-                                  const float* w, int rows, int dim, float eps, float mult, hipStream_t stream) {
+                                  const float* w, int rows, int dim, float eps, float mult, const float* next_w, float next_eps,
+                                  void* next_out, int next_dtype, hipStream_t stream) {
     if (rows <= 0) return 0;
-    if (dim <= 0 || (b != nullptr && (wa == nullptr || wb == nullptr))) return (int)hipErrorInvalidValue;
-    if (b) post_norm_add_kernel<true><<<rows, 256, 0, stream>>>(x, a, wa, b, wb, w, dim, eps, mult);
-    else post_norm_add_kernel<false><<<rows, 256, 0, stream>>>(x, a, nullptr, nullptr, nullptr, w, dim, eps, mult);
+    if (dim <= 0 || (b != nullptr && (wa == nullptr || wb == nullptr)) || (next_w != nullptr && next_out == nullptr))
+        return (int)hipErrorInvalidValue;
+    if (next_dtype == DT_F32) {
+        if (b) launch_post_norm_add<true, float>(x, a, wa, b, wb, w, rows, dim, eps, mult, next_w, next_eps, (float*)next_out, stream);
+        else launch_post_norm_add<false, float>(x, a, nullptr, nullptr, nullptr, w, rows, dim, eps, mult, next_w, next_eps, (float*)next_out, stream);
+    } else {
+        if (b) launch_post_norm_add<true, bf16_t>(x, a, wa, b, wb, w, rows, dim, eps, mult, next_w, next_eps, (bf16_t*)next_out, stream);
+        else launch_post_norm_add<false, bf16_t>(x, a, nullptr, nullptr, nullptr, w, rows, dim, eps, mult, next_w, next_eps, (bf16_t*)next_out, stream);
+    }
     return CISR_LAUNCH_CHECK();
 }
 

@@ -151,35 +151,51 @@ extern "C" int cisr_decay_gate(const float* z, int ld, const float* bias, float*
 //   u = y[t, i] + (skip ? skip[i / skip_span] * x[t * ldx + i] : 0)
 //   GATE_FIRST:  u *= silu(gate[t * ldg + i]);  out = u / rms(part) * w[shared ? d : i]
 //   else:        out = u / rms(part) * w[shared ? d : i] * silu(gate[t * ldg + i])
-// A block of NT threads a (row, part): a wave for parts of up to 256 elements, four waves for longer ones; the part is
-// read twice.
-template <typename T, bool GATE_FIRST, int NT>
+// A block of NT threads a (row, part): a wave for parts of up to 256 elements, four waves up to 2,048, sixteen beyond.
+// KEEP: the part's elements (after the skip term and the gate before the norm) wait in LDS for their scale, so every
+// input is read once; else (parts of more than 12,288 elements) they are made a second time.
+template <typename T, bool GATE_FIRST, int NT, bool KEEP>
 __global__ void __launch_bounds__(NT)
 group_norm_gate_kernel(const float* __restrict__ y, const float* __restrict__ gate, int ldg, const float* __restrict__ w,
                        int shared, const float* __restrict__ skip, int skip_span, const float* __restrict__ x, int ldx,
                        T* __restrict__ out, int size, float eps) {
     __shared__ float red[NT / WAVE];
+    extern __shared__ float kept[];
     const int t = blockIdx.x, g = blockIdx.y, groups = gridDim.y, lane = threadIdx.x;
     const size_t base = (size_t)t * groups * size + (size_t)g * size;
     const int col0 = g * size;
-    float ss = 0.f;
-    for (int d = lane; d < size; d += NT) {
+    auto element = [&](int d) {
         float u = y[base + d];
         if (skip) u += skip[(col0 + d) / skip_span] * x[(size_t)t * ldx + col0 + d];
         if (GATE_FIRST) { const float z = gate[(size_t)t * ldg + col0 + d]; u *= z / (1.0f + expf(-z)); }
+        return u;
+    };
+    float ss = 0.f;
+    for (int d = lane; d < size; d += NT) {
+        const float u = element(d);
+        if (KEEP) kept[d] = u;
         ss += u * u;
     }
     const float scale = 1.0f / sqrtf((NT == WAVE ? wave_sum(ss) : block_sum<NT>(ss, red)) / (float)size + eps);
     for (int d = lane; d < size; d += NT) {
-        float u = y[base + d];
-        if (skip) u += skip[(col0 + d) / skip_span] * x[(size_t)t * ldx + col0 + d];
-        const float z = gate[(size_t)t * ldg + col0 + d];
-        const float s = z / (1.0f + expf(-z));
-        if (GATE_FIRST) u *= s;
-        u *= scale * w[shared ? d : col0 + d];
-        if (!GATE_FIRST) u *= s;
+        float u = (KEEP ? kept[d] : element(d)) * scale * w[shared ? d : col0 + d];     // (a thread reads back what it wrote)
+        if (!GATE_FIRST) { const float z = gate[(size_t)t * ldg + col0 + d]; u *= z / (1.0f + expf(-z)); }
         store_f32(out + base + d, u);
     }
+}
+
+template <typename T, bool GATE_FIRST>
+static void launch_group_norm_gate(const float* y, const float* gate, int ldg, const float* w, int shared, const float* skip,
+                                   int skip_span, const float* x, int ldx, T* out, int rows, int groups, int size, float eps,
+                                   hipStream_t stream) {
+    const dim3 grid(rows, groups);
+    const size_t lds = (size_t)size * sizeof(float);
+#define GNG(NT, KEEP) group_norm_gate_kernel<T, GATE_FIRST, NT, KEEP><<<grid, NT, KEEP ? lds : 0, stream>>>(y, gate, ldg, w, shared, skip, skip_span, x, ldx, out, size, eps)
+    if (size <= 256) GNG(64, true);
+    else if (size <= 2048) GNG(256, true);
+    else if (size <= 12288) GNG(1024, true);
+    else GNG(1024, false);
+#undef GNG
 }
 
 extern "C" int cisr_group_norm_gate(const float* y, const float* gate, int ldg, const float* w, int shared, const float* skip,
@@ -187,13 +203,12 @@ extern "C" int cisr_group_norm_gate(const float* y, const float* gate, int ldg, 
                                     float eps, int gate_first, int dtype, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (groups <= 0 || groups > 65535 || size <= 0 || (skip && (skip_span <= 0 || !x))) return (int)hipErrorInvalidValue;
-    const dim3 grid(rows, groups);
-#define GNG(T, GF) do { \
-        if (size <= 256) group_norm_gate_kernel<T, GF, 64><<<grid, 64, 0, stream>>>(y, gate, ldg, w, shared, skip, skip_span, x, ldx, (T*)out, size, eps); \
-        else group_norm_gate_kernel<T, GF, 256><<<grid, 256, 0, stream>>>(y, gate, ldg, w, shared, skip, skip_span, x, ldx, (T*)out, size, eps); \
-    } while (0)
-    if (dtype == DT_F32) { if (gate_first) GNG(float, true); else GNG(float, false); }
-    else { if (gate_first) GNG(bf16_t, true); else GNG(bf16_t, false); }
-#undef GNG
+    if (dtype == DT_F32) {
+        if (gate_first) launch_group_norm_gate<float, true>(y, gate, ldg, w, shared, skip, skip_span, x, ldx, (float*)out, rows, groups, size, eps, stream);
+        else launch_group_norm_gate<float, false>(y, gate, ldg, w, shared, skip, skip_span, x, ldx, (float*)out, rows, groups, size, eps, stream);
+    } else {
+        if (gate_first) launch_group_norm_gate<bf16_t, true>(y, gate, ldg, w, shared, skip, skip_span, x, ldx, (bf16_t*)out, rows, groups, size, eps, stream);
+        else launch_group_norm_gate<bf16_t, false>(y, gate, ldg, w, shared, skip, skip_span, x, ldx, (bf16_t*)out, rows, groups, size, eps, stream);
+    }
     return CISR_LAUNCH_CHECK();
 }

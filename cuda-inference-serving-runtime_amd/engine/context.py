@@ -70,6 +70,7 @@ class StepContext:
         # part that was told it may (`next_norm`), taken by the norm that reads the rows next (or settled)
         self.unfinished = None
         self.next_norm = None     # the norm that reads the residual stream after the block that runs now, if known
+        self.normed = None        # (norm part, residual rows, normed rows): a block made its follower's first norm on the way
         self.layer_tap = getattr(runner, "layer_tap", None)   # callable(schedule index, residual rows) after every layer run, or None
         self.capturing = False    # the step is being recorded into a graph: launches only
         self.owner = None         # key of the captured program this step belongs to, if any
@@ -118,6 +119,17 @@ class StepContext:
             raise RuntimeError("the unfinished product belongs to other rows")
         partials, self.unfinished = self.unfinished[1], None
         return partials
+
+    def leave_normed(self, norm, rows, normed):
+        """`normed` = norm(rows) is made already: the block that runs next takes it instead of running its first norm."""
+        self.normed = (norm, rows, normed)
+
+    def take_normed(self, norm, rows):
+        """The rows that `norm` would make of `rows`, if the block before made them on its way; else None."""
+        got, self.normed = self.normed, None
+        if got is not None and got[0] is norm and got[1].data_ptr() == rows.data_ptr():
+            return got[2]
+        return None
 
     def settle(self, rows):
         """Add what `rows` lack, if anything: before a reader that cannot do it itself."""

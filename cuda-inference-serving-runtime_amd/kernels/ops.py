@@ -66,7 +66,7 @@ def _declare(h):
         "cisr_qkv_rope_wide": [p, i, p, i, p, i, i, i, p, p, p, p, p, p, i, i, i, i, i, p, C.c_longlong, p],
         "cisr_gemm_merged_bf16": [p, p, i, i, i, p, i, p, i, p, i, i, i, p],
         "cisr_gemm_merged_ok": [i, i, i, i, i],
-        "cisr_post_norm_add": [p, p, p, p, p, p, i, i, f, f, p],
+        "cisr_post_norm_add": [p, p, p, p, p, p, i, i, f, f, p, f, p, i, p],
         "cisr_glu_clamped": [p, p, i, i, f, f, f, i, p],
         "cisr_qk_norm_scatter": [p, i, p, p, p, p, p, p, i, i, i, i, i, i, i, f, i, p],
         "cisr_head_gate": [p, p, i, p, i, i, i, i, i, p],
@@ -826,10 +826,11 @@ def take_tokens(tokens, source, sampled):
 
 # -- layers that norm a sublayer's output, clamped gates, normed and gated attention ----------------------------------
 
-def post_norm_add(x, y, weight, eps, mult, second=None):
+def post_norm_add(x, y, weight, eps, mult, second=None, following=None):
     """x += mult * rmsnorm(y) * weight, in place (all float, [T, H]).  With `second` = (y2, w1, w2) the row that is
     normed is (rmsnorm(y) w1 + rmsnorm(y2) w2) / 2: two sublayers side by side.  `weight` None: no outer norm,
-    x += mult * row."""
+    x += mult * row.  `following` = (weight float [H], eps, out [T, H] float or bf16): the norm that reads x next is made
+    by the same kernel, out = rmsnorm(x) * weight."""
     rows, dim = x.shape
     xp = _dev(x, "x", torch.float32)
     yp = _dev(y, "y", torch.float32, (rows, dim))
@@ -839,7 +840,12 @@ def post_norm_add(x, y, weight, eps, mult, second=None):
         y2, w1, w2 = second
         bp = _dev(y2, "y2", torch.float32, (rows, dim))
         ap, w2p = _dev(w1, "w1", torch.float32, (dim,)), _dev(w2, "w2", torch.float32, (dim,))
-    _check(lib().cisr_post_norm_add(xp, yp, ap, bp, w2p, wp, rows, dim, float(eps), float(mult), _stream()), "post_norm_add")
+    np_, neps, op, odt = None, 0.0, None, F32
+    if following is not None:
+        nw, neps, out = following
+        np_, op, odt = _dev(nw, "following weight", torch.float32, (dim,)), _dev(out, "following out", None, (rows, dim)), _storage(out, "following out")
+    _check(lib().cisr_post_norm_add(xp, yp, ap, bp, w2p, wp, rows, dim, float(eps), float(mult), np_, float(neps), op, odt,
+                                    _stream()), "post_norm_add")
     return x
 
 
@@ -934,9 +940,9 @@ def scan_piece(rows, decode_only):
 
 def scan_columns(runs, heads, cols):
     """Columns of the state that one wave of the linear scan owns (16, 8 or 4): fewer columns make more waves of the
-    same head, until the launch has about two waves for every SIMD of the GPU.  `runs`: segments, or pieces of them."""
+    same head, until the launch has about a wave for every SIMD of the GPU (wider tiles read the state in longer runs).  `runs`: segments, or pieces of them."""
     for width in (16, 8, 4):
-        if runs * heads * -(-cols // width) >= 2048 or width == 4:
+        if runs * heads * -(-cols // width) >= 1024 or width == 4:
             return width
 
 

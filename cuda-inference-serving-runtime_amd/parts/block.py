@@ -77,16 +77,18 @@ class NormedMean:
         self.first, self.first_weight, self.second, self.second_weight, self.eps = first, first_weight, second, second_weight, eps
 
 
-def add_sublayer(residual, result, norm, mult, eps=None):
-    """residual += mult * norm(result) (norm None: mult * result); `result` float rows or a NormedMean."""
+def add_sublayer(residual, result, norm, mult, eps=None, following=None):
+    """residual += mult * norm(result) (norm None: mult * result); `result` float rows or a NormedMean.
+    `following` = (norm part, out): the RMS norm that reads the residual stream next is made by the same kernel."""
     weight = None if norm is None else norm.weight
     eps = norm.eps if norm is not None else eps
+    then = None if following is None else (following[0].weight, following[0].eps, following[1])
     if isinstance(result, NormedMean):
         if eps is not None and eps != result.eps:
             raise ValueError("the norms inside a mean of two results and the norm around it must share their eps (one kernel)")
         return ops.post_norm_add(residual, result.first, weight, result.eps, mult,
-                                 second=(result.second, result.first_weight, result.second_weight))
-    return ops.post_norm_add(residual, result, weight, 0.0 if eps is None else eps, mult)
+                                 second=(result.second, result.first_weight, result.second_weight), following=then)
+    return ops.post_norm_add(residual, result, weight, 0.0 if eps is None else eps, mult, following=then)
 
 
 class SandwichBlock(Part):
@@ -139,14 +141,37 @@ class SandwichBlock(Part):
     def first_norm(self):
         return self.mixer_norm
 
+    @staticmethod
+    def _plain_rms(norm):
+        return norm is not None and getattr(norm, "fusable_as", None) == "rms"
+
     def forward(self, residual, ctx, site):
+        # the kernel that adds a sublayer's result also makes the norm that reads the residual stream next, where that
+        # is an RMS norm over all rows: this block's second norm, or the following block's first (ctx.next_norm), which
+        # finds its rows waiting in ctx.normed
+        after = ctx.next_norm
         ctx.next_norm = None          # (no product of this block is left to a later norm)
-        h = self.mixer_norm.forward(residual, ctx)
-        ctx.settle(residual)
-        add_sublayer(residual, self.mixer.output(h, ctx, site), self.mixer_post, self.mult)
-        if self.ffn is not None:
-            h = self.ffn_norm.forward(residual, ctx)
-            add_sublayer(residual, self.ffn.output(h, ctx), self.ffn_post, self.mult)
+        h = ctx.take_normed(self.mixer_norm, residual)
+        if h is None:
+            h = self.mixer_norm.forward(residual, ctx)
+            ctx.settle(residual)
+        T = residual.shape[0]
+        last = self.ffn is None
+
+        def following(norm, tag):
+            return (norm, ctx.buffer(tag, (T, residual.shape[1]), ctx.dtype)) if self._plain_rms(norm) else None
+
+        then = following(after if last else self.ffn_norm, "norm.ahead" if last else "norm.inside")
+        add_sublayer(residual, self.mixer.output(h, ctx, site), self.mixer_post, self.mult, following=then)
+        if last:
+            if then is not None:
+                ctx.leave_normed(after, residual, then[1])
+            return residual
+        h = then[1] if then is not None else self.ffn_norm.forward(residual, ctx)
+        then = following(after, "norm.ahead")
+        add_sublayer(residual, self.ffn.output(h, ctx), self.ffn_post, self.mult, following=then)
+        if then is not None:
+            ctx.leave_normed(after, residual, then[1])
         return residual
 
 
