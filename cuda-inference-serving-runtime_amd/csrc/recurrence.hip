@@ -44,7 +44,7 @@ extern "C" int cisr_linear_scan(const float* q, int ldq, const float* k, int ldk
         return (int)hipErrorInvalidValue;
     ScanArgs p{q, ldq, k, ldk, v, ldv, a, lda, vs, ldvs, out, ldo, state, slot_stride, seg_start, state_slots, R, C, share, heads,
                q_scale, piece, piece > 0 ? (rows + piece - 1) / piece : 1, 0, carry, carry_decay};
-    if ((C + cols - 1) / cols > 65535 || R > 256) return (int)hipErrorInvalidValue;
+    if ((C + cols - 1) / cols > 65535 || R > 256 || (piece > 0 && segments > 65535)) return (int)hipErrorInvalidValue;
     if (cols == 4) return cisr_scan_launch_c4(p, segments, vec, stream);
     if (cols == 8) return cisr_scan_launch_c8(p, segments, vec, stream);
     return cisr_scan_launch_c16(p, segments, vec, stream);
@@ -135,6 +135,30 @@ __global__ void decay_gate_kernel(const float* __restrict__ z, int ld, const flo
     const int c = (int)(i % cols);
     const float u = z[t * ld + c] + (bias ? bias[c] : 0.f);
     a[i] = expf((fminf(u, 0.f) - log1pf(expf(-fabsf(u)))) * inv_tau);
+}
+
+// The same with z = up . low made on the way: z[t, c] = sum_r up[c * rank + r] * low[t * ld + r] (the second half of a
+// low-rank projection; the first half came out of the mixer's fused input product).
+__global__ void decay_gate_low_rank_kernel(const float* __restrict__ low, int ld, int rank, const float* __restrict__ up,
+                                           const float* __restrict__ bias, float* __restrict__ a, int cols, size_t n, float inv_tau) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const size_t t = i / cols;
+    const int c = (int)(i % cols);
+    const float* lo = low + t * ld;
+    const float* w = up + (size_t)c * rank;
+    float u = bias ? bias[c] : 0.f;
+    for (int r = 0; r < rank; ++r) u += w[r] * lo[r];
+    a[i] = expf((fminf(u, 0.f) - log1pf(expf(-fabsf(u)))) * inv_tau);
+}
+
+extern "C" int cisr_decay_gate_low_rank(const float* low, int ld, int rank, const float* up, const float* bias, float* a,
+                                        int rows, int cols, float tau, hipStream_t stream) {
+    const size_t n = (size_t)rows * cols;
+    if (n == 0) return 0;
+    if (!(tau > 0.f) || rank <= 0) return (int)hipErrorInvalidValue;
+    decay_gate_low_rank_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(low, ld, rank, up, bias, a, cols, n, 1.0f / tau);
+    return CISR_LAUNCH_CHECK();
 }
 
 extern "C" int cisr_decay_gate(const float* z, int ld, const float* bias, float* a, int rows, int cols, float tau,

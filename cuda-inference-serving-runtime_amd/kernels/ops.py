@@ -908,6 +908,7 @@ def _rec():
             "cisr_linear_scan": [p, i, p, i, p, i, p, i, i, p, i, p, i, p, ll, p, p, i, i, i, i, i, f, i, i, i, p, p, p],
             "cisr_conv_silu": [p, i, i, p, p, p, ll, p, p, p, p, i, i, i, i, i, i, p, p, p, p, p],
             "cisr_decay_gate": [p, i, p, p, i, i, f, p],
+            "cisr_decay_gate_low_rank": [p, i, i, p, p, p, i, i, f, p],
             "cisr_group_norm_gate": [p, p, i, p, i, p, i, p, i, p, i, i, i, f, i, i, p],
         }
         for name, args in sig.items():
@@ -1035,6 +1036,18 @@ def decay_gate(z, bias, out, tau):
     zp, ld = _rows_of(z, "z")
     _check(_rec().cisr_decay_gate(zp, ld, None if bias is None else _dev(bias, "bias", torch.float32, (n,)),
                                   _dev(out, "out", torch.float32, (T, n)), T, n, float(tau), _stream()), "decay_gate")
+    return out
+
+
+def decay_gate_low_rank(low, up, bias, out, tau):
+    """out = sigmoid(low . up^T + bias)^(1 / tau) in float: low a float view [T, rank] (the first half of a low-rank
+    projection), up float [N, rank], bias float [N] or None, out float [T, N]."""
+    T, rank = low.shape
+    n = up.shape[0]
+    lp, ld = _rows_of(low, "low")
+    _check(_rec().cisr_decay_gate_low_rank(lp, ld, rank, _dev(up, "up", torch.float32, (n, rank)),
+                                           None if bias is None else _dev(bias, "bias", torch.float32, (n,)),
+                                           _dev(out, "out", torch.float32, (T, n)), T, n, float(tau), _stream()), "decay_gate_low_rank")
     return out
 
 

@@ -67,26 +67,28 @@ class GatedLinearAttention(Mixer):
                 TensorSpec(self._tensor("bias"), (K,))]
 
     def bind(self, tensors, dtype):
-        self.w_in = torch.cat([matrix_operand(tensors[self._tensor(p)], dtype) for p in ("q", "k", "v", "gate")], dim=0).contiguous()
-        self.w_down, self.w_up = matrix_operand(tensors[self._tensor("down")], dtype), matrix_operand(tensors[self._tensor("up")], dtype)
-        if self.w_down.shape[0] != self.w_up.shape[1]:
+        # one product for q, k, v, the gate and the first half of the decay's low-rank projection; its second half is a
+        # few multiplications a decay, done in float by the kernel that makes the decays
+        parts = [matrix_operand(tensors[self._tensor(p)], dtype) for p in ("q", "k", "v", "gate", "down")]
+        self.low_rank = parts[-1].shape[0]
+        self.w_up = _float(tensors[self._tensor("up")])
+        if self.low_rank != self.w_up.shape[1]:
             raise ValueError(f"{self.name}: the decay's projections disagree about their inner size "
-                             f"({self.w_down.shape[0]} and {self.w_up.shape[1]})")
+                             f"({self.low_rank} and {self.w_up.shape[1]})")
+        self.w_in = torch.cat(parts, dim=0).contiguous()
         self.w_out = matrix_operand(tensors[self._tensor("o")], dtype)
         self.norm_weight, self.bias = _float(tensors[self._tensor("norm")]), _float(tensors[self._tensor("bias")])
 
     def output(self, h, ctx, site):
         T = h.shape[0]
         K, V = self.heads * self.dim, self.heads * self.vdim
-        proj = ops.gemm(h, self.w_in, ctx.buffer("gla.proj", (T, 2 * K + 2 * V), torch.float32), scratch=ctx.scratch)
-        low = ops.gemm(h, self.w_down, ctx.buffer("gla.low", (T, self.w_down.shape[0]), ctx.dtype), scratch=ctx.scratch)
-        z = ops.gemm(low, self.w_up, ctx.buffer("gla.decay", (T, K), torch.float32), scratch=ctx.scratch)
-        decay = ops.decay_gate(z, self.bias, z, self.tau)          # (in place: an element is read and written by one thread)
+        proj = ops.gemm(h, self.w_in, ctx.buffer("gla.proj", (T, self.w_in.shape[0]), torch.float32), scratch=ctx.scratch)
+        decay = ops.decay_gate_low_rank(proj[:, 2 * K + 2 * V:], self.w_up, self.bias, ctx.buffer("gla.decay", (T, K), torch.float32), self.tau)
         state = ctx.cache.state_storage[site]
         o = ctx.buffer("gla.o", (T, V), torch.float32)
         _scan(ctx, "gla", proj[:, :K], proj[:, K:2 * K], proj[:, 2 * K:2 * K + V], decay, o, state.view(state.shape[0], -1),
               self.heads, self.dim, self.vdim, q_scale=self.dim ** -0.5)
-        act = ops.group_norm_gate(o, proj[:, 2 * K + V:], self.norm_weight, ctx.buffer("gla.act", (T, V), ctx.dtype),
+        act = ops.group_norm_gate(o, proj[:, 2 * K + V:2 * K + 2 * V], self.norm_weight, ctx.buffer("gla.act", (T, V), ctx.dtype),
                                   self.heads, self.eps, gate_first=False, shared_weight=True)
         return ops.gemm(act, self.w_out, ctx.buffer("gla.y", (T, self.hidden), torch.float32), scratch=ctx.scratch)
 
