@@ -62,4 +62,19 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
     return total;
 }
 
+// The law of a gated activation act(gate, up), the epilogue of a product over [gate; up]:
+//   limit <= 0:  silu(g) u
+//   limit > 0:   g' sigmoid(slope g') (u' + shift) with g' = min(g, limit), u' = clamp(u, -limit, limit)
+// A struct of zeros is the first law.
+struct GateLaw { float limit, slope, shift; };
+
+__device__ __forceinline__ float gated_activation(float g, float u, const GateLaw& law) {
+    if (law.limit > 0.f) {
+        g = fminf(g, law.limit);
+        u = fminf(fmaxf(u, -law.limit), law.limit);
+        return g / (1.0f + expf(-law.slope * g)) * (u + law.shift);
+    }
+    return g / (1.0f + expf(-g)) * u;
+}
+
 #define CISR_LAUNCH_CHECK() ((int)hipGetLastError())

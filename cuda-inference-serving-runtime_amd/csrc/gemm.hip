@@ -130,7 +130,7 @@ __host__ __device__ inline int patch_side(int tiles) {
 template <int TM, int TN, int BK, typename TC, bool VEC, bool SWIGLU = false, int WM = 2>
 __global__ void __launch_bounds__(WM * 128)
 gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
-                 TC* C, int ldc, const float* R, int ldr, int M, int N, int K, int dual_off = 0) {
+                 TC* C, int ldc, const float* R, int ldr, int M, int N, int K, int dual_off = 0, GateLaw law = {}) {
     static_assert(!SWIGLU || (TN % 2 == 0 && VEC), "the activation pairs column tiles");
     constexpr int BM = WM * TM * 16, BN = 2 * TN * 16, NT = WM * 128;   // WM x 2 waves
     constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;           // output columns a block covers
@@ -251,7 +251,7 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
                 for (int e = 0; e < 4; ++e) {
                     const int m = m0 + wm * TM * 16 + i * 16 + g * 4 + e;
                     const float gq = bf16_to_f32(f32_to_bf16(acc[i][j][e])), uq = bf16_to_f32(f32_to_bf16(acc[i][j + TN / 2][e]));
-                    if (m < M) store_f32(C + (size_t)m * ldc + n, gq / (1.0f + expf(-gq)) * uq);
+                    if (m < M) store_f32(C + (size_t)m * ldc + n, gated_activation(gq, uq, law));
                 }
             }
         return;
@@ -317,18 +317,32 @@ static int launch_bf16(const bf16_t* A, int lda, const bf16_t* W, int ldw, void*
 // 16-byte aligned rows with K % 8 == 0.
 template <int TM, int TN, int BK, int WM = 2>
 static int launch_bf16_swiglu(const bf16_t* A, int lda, const bf16_t* W, int ldw, bf16_t* C, int ldc, int M, int N, int K,
-                              int dual_off, hipStream_t stream) {
+                              int dual_off, GateLaw law, hipStream_t stream) {
     constexpr int BM = WM * TM * 16, BN_OUT = TN * 16;
     const long long slots = tile_slots((M + BM - 1) / BM, (N + BN_OUT - 1) / BN_OUT);
     if (slots > (1ll << 30)) return (int)hipErrorInvalidValue;
     dim3 grid((unsigned)((slots + 7) / 8 * 8));
-    gemm_bf16_kernel<TM, TN, BK, bf16_t, true, true, WM><<<grid, WM * 128, 0, stream>>>(A, lda, W, ldw, C, ldc, nullptr, 0, M, N, K, dual_off);
+    gemm_bf16_kernel<TM, TN, BK, bf16_t, true, true, WM><<<grid, WM * 128, 0, stream>>>(A, lda, W, ldw, C, ldc, nullptr, 0, M, N, K, dual_off, law);
     return CISR_LAUNCH_CHECK();
 }
 
 // `tile`: 0 picks by the rule below; TM * 100 + TN * 10 + WM asks for that block tile (a tile that is not built: an error).
+static int swiglu_tile_entry(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N, int K,
+                             int dual_off, int tile, GateLaw law, hipStream_t stream);
+
 extern "C" int cisr_gemm_bf16_swiglu_tile(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N, int K,
                                           int dual_off, int tile, hipStream_t stream) {
+    return swiglu_tile_entry(A, lda, W, ldw, C, ldc, M, N, K, dual_off, tile, GateLaw{}, stream);
+}
+
+// The same with the gated activation's law given: see GateLaw.
+extern "C" int cisr_gemm_bf16_gated(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N, int K,
+                                    int dual_off, float limit, float slope, float shift, hipStream_t stream) {
+    return swiglu_tile_entry(A, lda, W, ldw, C, ldc, M, N, K, dual_off, 0, GateLaw{limit, slope, shift}, stream);
+}
+
+static int swiglu_tile_entry(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N, int K,
+                             int dual_off, int tile, GateLaw law, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (K <= 0 || K % 8 || lda % 8 || ldw % 8 || ((uintptr_t)A) % 16 || ((uintptr_t)W) % 16 || dual_off < N)
         return (int)hipErrorInvalidValue;
@@ -341,7 +355,7 @@ extern "C" int cisr_gemm_bf16_swiglu_tile(const void* A, int lda, const void* W,
         else tile = 222;
     }
 #define SWIGLU_TILE(TM, TN, WM) \
-    case TM * 100 + TN * 10 + WM: return launch_bf16_swiglu<TM, TN, 64, WM>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, dual_off, stream);
+    case TM * 100 + TN * 10 + WM: return launch_bf16_swiglu<TM, TN, 64, WM>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, dual_off, law, stream);
     switch (tile) {
         SWIGLU_TILE(1, 2, 2) SWIGLU_TILE(2, 2, 2) SWIGLU_TILE(4, 2, 2) SWIGLU_TILE(4, 4, 2)
     }

@@ -13,6 +13,7 @@ struct SkinnyArgs {
     const float* R; int ldr;           // residual (EPI_STORE, float C only)
     int M, N, K;
     int dual_off;                      // EPI_SWIGLU
+    GateLaw law;                       // EPI_SWIGLU: the activation's law (zeros: silu(g) u)
     // NORM
     const float* norm_w; float eps; const int* rows;
     // EPI_ROPE

@@ -35,6 +35,7 @@ struct WideArgs {
     int units;                  // 16-row units of W
     int slices;                 // slices of K: SPW / 2 rounds of NW pairs of 32-wide k-steps each
     int dual_off;               // two blocks of W this many rows apart (SwiGLU), or 0
+    GateLaw law;                // the gated activation's law (zeros: silu(g) u)
     int leave_partials;         // several slices: no second kernel, the caller's next kernel adds the partial sums
     // the fused q/k/v projection (head_dim > 0): C is q, bf16 [M, heads * head_dim]
     const int* positions; const int* slots; const float* cos_tab; const float* sin_tab;
@@ -79,7 +80,7 @@ __device__ __forceinline__ void wide_finish(const WideArgs& p, int m, int n, flo
     if (NB == 2) {
         // gate and up are rounded to bf16 before the activation, as the two-kernel path does
         const float gq = bf16_to_f32(f32_to_bf16(v)), uq = bf16_to_f32(f32_to_bf16(u));
-        v = gq / (1.0f + expf(-gq)) * uq;
+        v = gated_activation(gq, uq, p.law);
     }
     if (p.R) v += p.R[(size_t)m * p.ldr + n];
     if (p.out_dtype == DT_F32) ((float*)p.C)[(size_t)m * p.ldc + n] = v;
@@ -321,7 +322,7 @@ static bool wide_aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 static int wide_entry(const void* A, int lda, const void* W, int ldw, void* C, int ldc, const float* R, int ldr, int M, int N,
                       int K, int out_dtype, int dual_off, float* workspace, long long workspace_floats, bool plan_only,
-                      long long* need, hipStream_t stream, bool leave_partials = false) {
+                      long long* need, hipStream_t stream, bool leave_partials = false, GateLaw law = {}) {
     if (need) *need = 0;
     if (M <= 0 || N <= 0) return 0;
     if (M > 64 || K < 8 || K % 8 || lda % 8 || ldw % 8 || dual_off < 0 || workspace_floats < 0 ||
@@ -330,6 +331,7 @@ static int wide_entry(const void* A, int lda, const void* W, int ldw, void* C, i
     if (!plan_only && (!wide_aligned16(A) || !wide_aligned16(W) || (!C && !leave_partials))) return (int)hipErrorInvalidValue;
     WideArgs a = {};
     a.leave_partials = leave_partials;
+    a.law = law;
     a.A = (const bf16_t*)A; a.lda = lda; a.W = (const bf16_t*)W; a.ldw = ldw; a.C = C; a.ldc = ldc; a.out_dtype = out_dtype;
     a.R = R; a.ldr = ldr; a.P = workspace; a.M = M; a.N = N; a.K = K; a.units = (N + 15) / 16; a.dual_off = dual_off;
     return dual_off > 0 ? wide_dispatch<2, false>(a, (size_t)workspace_floats, plan_only, need, stream)
@@ -374,6 +376,15 @@ extern "C" int cisr_gemm_wide_bf16(const void* A, int lda, const void* W, int ld
                                    long long workspace_floats, hipStream_t stream) {
     return wide_entry(A, lda, W, ldw, C, ldc, R, ldr, M, N, K, out_dtype, dual_off, workspace, workspace_floats, false,
                       nullptr, stream);
+}
+
+// The same with the gated activation's law given (dual_off > 0): see GateLaw.
+extern "C" int cisr_gemm_wide_bf16_gated(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N, int K,
+                                         int dual_off, float limit, float slope, float shift, float* workspace,
+                                         long long workspace_floats, hipStream_t stream) {
+    if (dual_off <= 0) return (int)hipErrorInvalidValue;
+    return wide_entry(A, lda, W, ldw, C, ldc, nullptr, 0, M, N, K, DT_BF16, dual_off, workspace, workspace_floats, false,
+                      nullptr, stream, false, GateLaw{limit, slope, shift});
 }
 
 // The first pass alone, for a product that is cut into several slices (cisr_gemm_wide_workspace(M, N, K, 0) > 0; an

@@ -325,7 +325,7 @@ gemv_kernel(SkinnyArgs p, int units, int per_wave) {
             const float v1 = v[R - 1] * scale;
             // the two-kernel path rounds gate and up to bf16 before the activation; do the same
             const float gq = bf16_to_f32(f32_to_bf16(v0)), uq = bf16_to_f32(f32_to_bf16(v1));
-            ((bf16_t*)p.C)[(size_t)m * p.ldc + u] = f32_to_bf16(gq / (1.0f + expf(-gq)) * uq);
+            ((bf16_t*)p.C)[(size_t)m * p.ldc + u] = f32_to_bf16(gated_activation(gq, uq, p.law));
         } else {
             float v1 = v[R - 1] * scale;
             const int D = p.head_dim, half = D / 2, sh = u / half, i = u % half;

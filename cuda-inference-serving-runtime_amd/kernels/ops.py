@@ -66,6 +66,9 @@ def _declare(h):
         "cisr_qkv_rope_wide": [p, i, p, i, p, i, i, i, p, p, p, p, p, p, i, i, i, i, i, p, C.c_longlong, p],
         "cisr_gemm_merged_bf16": [p, p, i, i, i, p, i, p, i, p, i, i, i, p],
         "cisr_gemm_merged_ok": [i, i, i, i, i],
+        "cisr_gemm_skinny_bf16_gated": [p, i, p, i, p, i, i, i, i, i, f, f, f, p],
+        "cisr_gemm_wide_bf16_gated": [p, i, p, i, p, i, i, i, i, i, f, f, f, p, C.c_longlong, p],
+        "cisr_gemm_bf16_gated": [p, i, p, i, p, i, i, i, i, i, f, f, f, p],
         "cisr_post_norm_add": [p, p, p, p, p, p, i, i, f, f, p, f, p, i, p],
         "cisr_glu_clamped": [p, p, i, i, f, f, f, i, p],
         "cisr_qk_norm_scatter": [p, i, p, p, p, p, p, p, i, i, i, i, i, i, i, f, i, p],
@@ -587,8 +590,9 @@ def gemm_normed(x, norm, w, out):
     return out
 
 
-def gemm_swiglu(a, w_gate_up, out, gate_up=None, norm=None, scratch=None):
-    """out[M, I] = silu(a . Wg^T) * (a . Wu^T) with w_gate_up = [Wg; Wu] ([2I, K]).
+def gemm_swiglu(a, w_gate_up, out, gate_up=None, norm=None, scratch=None, law=None):
+    """out[M, I] = silu(a . Wg^T) * (a . Wu^T) with w_gate_up = [Wg; Wu] ([2I, K]); with `law` = (limit, slope, shift)
+    the activation is g sigmoid(slope g) (u + shift), g = min(gate, limit), u = clamp(up, -limit, limit) instead.
     Few rows of bf16 run one fused weight-streaming kernel (with `norm` = (weight, eps, None), `a` is the float
     residual and RMSNorm is fused too); otherwise the product goes to `gate_up` [M, 2I] and the activation is
     a second kernel.  `scratch`: the ScratchPool of the caller's steps."""
@@ -598,6 +602,8 @@ def gemm_swiglu(a, w_gate_up, out, gate_up=None, norm=None, scratch=None):
     if k != k2 or two_i % 2 or tuple(out.shape) != (m, inter) or not out.is_contiguous():
         raise KernelError("gemm_swiglu: shapes do not fit")
     if norm is not None:
+        if law is not None:
+            raise KernelError("gemm_swiglu: the fused norm comes with the silu law only")
         wp, eps, rp, _ = _norm_args(a, norm, k)
         if not fused_norm_ok(a, w_gate_up, m) or out.dtype != torch.bfloat16:
             raise KernelError("gemm_swiglu: shape not supported by the fused kernel")
@@ -607,10 +613,30 @@ def gemm_swiglu(a, w_gate_up, out, gate_up=None, norm=None, scratch=None):
         return out
     if out.dtype != a.dtype or a.dtype != w_gate_up.dtype:
         raise KernelError("gemm_swiglu: dtypes differ")
+    activate = swiglu if law is None else (lambda gu, o: glu_clamped(gu, o, *law))
     if a.dtype == torch.bfloat16 and library_ok(m, w_gate_up, gated=True) and a.is_contiguous():
         product = _scratch_bf16(scratch, a.device, m, two_i)
         torch.mm(a, w_gate_up.t(), out=product)
-        return swiglu(product, out)
+        return activate(product, out)
+    if swiglu_fused_ok(a, w_gate_up) and law is not None:
+        # the same kernels with the activation's law given
+        lim, slope, shift = (float(x) for x in law)
+        if m <= SKINNY_ROWS and wide_ok(m, w_gate_up, True, after_norm=True):
+            need = _wide_plan(m, inter, k, True)
+            if need < 0 or a.stride(0) % 8 or a.data_ptr() % 16:
+                raise KernelError("gemm_swiglu: shape not supported by the wide kernel")
+            work = _wide_workspace(scratch, a.device, need)
+            code = lib().cisr_gemm_wide_bf16_gated(a.data_ptr(), a.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0), out.data_ptr(),
+                                                   out.stride(0), m, inter, k, inter, lim, slope, shift,
+                                                   None if work is None else work.data_ptr(), 0 if work is None else work.numel(), _stream())
+        elif m <= SKINNY_ROWS:
+            code = lib().cisr_gemm_skinny_bf16_gated(a.data_ptr(), a.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0), out.data_ptr(),
+                                                     out.stride(0), m, inter, k, inter, lim, slope, shift, _stream())
+        else:
+            code = lib().cisr_gemm_bf16_gated(a.data_ptr(), a.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0), out.data_ptr(),
+                                              out.stride(0), m, inter, k, inter, lim, slope, shift, _stream())
+        _check(code, "gemm_swiglu")
+        return out
     if swiglu_fused_ok(a, w_gate_up):
         if m <= SKINNY_ROWS and wide_ok(m, w_gate_up, True, after_norm=True):
             return _gemm_wide(a, w_gate_up, out, None, True, "gemm_swiglu", scratch)
@@ -625,7 +651,7 @@ def gemm_swiglu(a, w_gate_up, out, gate_up=None, norm=None, scratch=None):
     if gate_up is None:
         raise KernelError("gemm_swiglu: this shape needs a buffer [M, 2I] for the product of gate and up")
     gemm(a, w_gate_up, gate_up, scratch=scratch)
-    return swiglu(gate_up, out)
+    return activate(gate_up, out)
 
 
 def qkv_rope_fused_ok(a, w, head_dim, cos, normed):

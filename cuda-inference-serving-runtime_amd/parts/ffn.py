@@ -78,8 +78,13 @@ class ClampedGLU(FeedForward):
     def output(self, h, ctx):
         """The feed-forward's result, float [T, hidden], without the residual sum."""
         T = h.shape[0]
-        gate_up = ops.gemm(h, self.w_gate_up, ctx.buffer("ffn.gate_up", (T, 2 * self.intermediate), ctx.dtype), scratch=ctx.scratch)
-        act = ops.glu_clamped(gate_up, ctx.buffer("ffn.act", (T, self.intermediate), ctx.dtype), self.limit, self.slope, self.shift)
+        law = (self.limit, self.slope, self.shift)
+        act = ctx.buffer("ffn.act", (T, self.intermediate), ctx.dtype)
+        if ops.swiglu_fused_ok(h, self.w_gate_up):
+            ops.gemm_swiglu(h, self.w_gate_up, act, scratch=ctx.scratch, law=law)      # the product and the activation are one kernel
+        else:
+            ops.gemm_swiglu(h, self.w_gate_up, act, gate_up=ctx.buffer("ffn.gate_up", (T, 2 * self.intermediate), ctx.dtype),
+                            scratch=ctx.scratch, law=law)
         return ops.gemm(act, self.w_down, ctx.buffer("ffn.out", (T, self.hidden), torch.float32), scratch=ctx.scratch)
 
     def forward(self, h, residual, ctx, norm=None):

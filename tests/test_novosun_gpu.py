@@ -211,6 +211,23 @@ def test_decay_gate_group_norm_gate_post_norm_and_clamped_gate():
         close(out.float().cpu().numpy(), P.clamped_glu(ref[:, :21], ref[:, 21:], 1.25), tol)
 
 
+@pytest.mark.parametrize("rows", [1, 3, 16, 40, 100])
+@pytest.mark.parametrize("inner, width", [(64, 48), (1024, 4096)])
+def test_clamped_gate_as_the_epilogue_of_the_product_over_gate_and_up(rows, inner, width):
+    """Every kernel that takes the product over [gate; up] (matrix-vector, narrow, skinny, wide, tiled) with the clamped
+    law, against the float product of the same operands (gate and up rounded to bfloat16 before the activation)."""
+    from runtime.kernels import ops
+    rng = np.random.default_rng(rows + inner)
+    a = dev(rng.standard_normal((rows, inner)), torch.bfloat16)
+    w = dev(rng.standard_normal((2 * width, inner)) * 2.0 / np.sqrt(inner), torch.bfloat16)
+    out = ops.gemm_swiglu(a, w, torch.zeros((rows, width), device=DEV, dtype=torch.bfloat16), law=(1.25, 1.702, 1.0))
+    gu = (a.float() @ w.float().T).to(torch.bfloat16).float().cpu().numpy()
+    want = P.clamped_glu(gu[:, :width], gu[:, width:], 1.25)
+    got = out.float().cpu().numpy()
+    assert np.abs(got - want).max() < 2e-2 * np.abs(want).max()       # (a bfloat16 step of gate or up moves the result this far)
+    assert np.sqrt(((got - want) ** 2).mean()) < 4e-3 * np.abs(want).max()
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads, kv_heads, dim, vdim", [(4, 2, 24, 16), (2, 2, 16, 40), (3, 1, 8, 8), (1, 1, 70, 130)])
 def test_normed_queries_and_keys_land_in_padded_heads_and_pages(dtype, heads, kv_heads, dim, vdim):
