@@ -1015,8 +1015,8 @@ def linear_scan(q, k, v, decay, out, state, seg_start, state_slots, heads, rows_
             raise KernelError("linear_scan: pieces need the carry buffers that scan_carry sizes")
         cp, dp = _dev(carry[0], "carry", torch.float32), _dev(carry[1], "carry_decay", torch.float32)
     cols = int(columns or scan_columns(-(-T // piece) if piece else segments, heads, Cc))
-    while -(-R // (64 // cols)) > 64:
-        cols *= 2          # (a lane holds at most 64 rows of its column)
+    while columns is None and cols > 4 and -(-R // (128 // cols)) > 16:
+        cols //= 2         # (at most 16 rows of its two columns a lane, where the tile can be narrower: registers)
     _check(_rec().cisr_linear_scan(qp, ldq, kp, ldk, vp, ldv, ap, lda, int(vec), sp, lds, op, ldo, state.data_ptr(),
                                    state.stride(0), _dev(seg_start, "seg_start", torch.int32, (segments + 1,)),
                                    _dev(state_slots, "state_slots", torch.int32, (segments,)), segments, heads, R, Cc,
