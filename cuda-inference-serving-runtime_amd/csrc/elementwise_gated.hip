@@ -96,10 +96,35 @@ __global__ void glu_clamped_kernel(const T* __restrict__ gu, T* __restrict__ act
     store_f32(act + i, g / (1.0f + expf(-slope * g)) * (u + shift));
 }
 
+// the same for bf16, eight elements a thread with 16-byte accesses (inter % 8 == 0, aligned pointers)
+__global__ void __launch_bounds__(256)
+glu_clamped_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ act, int inter8, size_t n8, GateLaw law) {
+    typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n8) return;
+    const size_t row = i / inter8;
+    const int col = (int)(i % inter8) * 8;
+    const bf16_t* base = gu + row * (size_t)(16 * inter8);
+    const u32x4_t g = *(const u32x4_t*)(base + col), u = *(const u32x4_t*)(base + 8 * inter8 + col);
+    const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
+    uint32_t out[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+        out[k] = pack_bf16x2(gated_activation(__uint_as_float(gw[k] << 16), __uint_as_float(uw[k] << 16), law),
+                             gated_activation(__uint_as_float(gw[k] & 0xffff0000u), __uint_as_float(uw[k] & 0xffff0000u), law));
+    *(u32x4_t*)(act + i * 8) = (u32x4_t){out[0], out[1], out[2], out[3]};
+}
+
 extern "C" int cisr_glu_clamped(const void* gu, void* act, int rows, int inter, float limit, float slope, float shift,
                                 int dtype, hipStream_t stream) {
     const size_t n = (size_t)rows * inter;
     if (n == 0) return 0;
+    if (dtype == DT_BF16 && limit > 0.f && inter % 8 == 0 && ((uintptr_t)gu) % 16 == 0 && ((uintptr_t)act) % 16 == 0) {
+        const size_t n8 = n / 8;
+        glu_clamped_bf16x8_kernel<<<(unsigned)((n8 + 255) / 256), 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)act, inter / 8, n8,
+                                                                                  GateLaw{limit, slope, shift});
+        return CISR_LAUNCH_CHECK();
+    }
     const unsigned blocks = (unsigned)((n + 255) / 256);
     if (dtype == DT_F32) glu_clamped_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)act, inter, n, limit, slope, shift);
     else glu_clamped_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)act, inter, n, limit, slope, shift);

@@ -203,12 +203,19 @@ def test_decay_gate_group_norm_gate_post_norm_and_clamped_gate():
     x = dev(x0)
     ops.post_norm_add(x, dev(a), None, 0.0, 1.0, second=(dev(b), dev(wa), dev(wb)))
     close(x.cpu().numpy(), x0 + 0.5 * (P.rmsnorm(a, wa, 0.0) + P.rmsnorm(b, wb, 0.0)))
-    gu = rng.standard_normal((T, 2 * 21)) * 3
-    for dtype, tol in ((torch.float32, 2e-5), (torch.bfloat16, 8e-3)):
-        operand = dev(gu, dtype)
-        out = ops.glu_clamped(operand, torch.zeros((T, 21), device=DEV, dtype=dtype), 1.25)
-        ref = operand.float().cpu().numpy()
-        close(out.float().cpu().numpy(), P.clamped_glu(ref[:, :21], ref[:, 21:], 1.25), tol)
+    for inter in (21, 24):                                 # (rows of a multiple of eight: 16-byte accesses)
+        gu = rng.standard_normal((T, 2 * inter)) * 3
+        for dtype, tol in ((torch.float32, 2e-5), (torch.bfloat16, 8e-3)):
+            operand = dev(gu, dtype)
+            out = ops.glu_clamped(operand, torch.zeros((T, inter), device=DEV, dtype=dtype), 1.25)
+            ref = operand.float().cpu().numpy()
+            close(out.float().cpu().numpy(), P.clamped_glu(ref[:, :inter], ref[:, inter:], 1.25), tol)
+    # the norm that reads the residual stream next, made on the way
+    x = dev(x0)
+    ahead = torch.zeros((T, H), device=DEV, dtype=torch.bfloat16)
+    ops.post_norm_add(x, dev(a), dev(wn), 1e-2, 0.3, following=(dev(wa), 1e-3, ahead))
+    close(x.cpu().numpy(), x0 + 0.3 * P.rmsnorm(a, wn, 1e-2))
+    close(ahead.float().cpu().numpy(), P.rmsnorm(x0 + 0.3 * P.rmsnorm(a, wn, 1e-2), wa, 1e-3), 8e-3)
 
 
 @pytest.mark.parametrize("rows", [1, 3, 16, 40, 100])
@@ -430,3 +437,27 @@ def test_greedy_generation_through_the_scheduler(folders, dtype, execution, over
                 assert row.max() - row[token] < 0.05 * (row.max() - row.min())
     engine.runner.cache.check()
     assert not engine.runner.cache.lengths, "every request gave back what it held"
+
+
+def test_command_line_serves_the_design(folders, tmp_path):
+    """`python -m runtime` chooses the design by config.json: requests of a file against a folder, in float32, give the
+    plain model's greedy tokens; the named configuration with random weights generates and reports its state slots."""
+    import json, os, subprocess, sys
+    from conftest import ROOT
+    cfg, w = P.read_folder(folders["p"])
+    requests = [{"key": "x", "prompt": [1, 2, 3, 4, 5, 6, 7], "max_new_tokens": 5}, {"key": "y", "prompt": [9], "max_new_tokens": 4}]
+    (tmp_path / "requests.json").write_text(json.dumps(requests))
+    env = dict(os.environ, PYTHONPATH=str(ROOT))
+    proc = subprocess.run([sys.executable, "-m", "runtime", "--checkpoint", str(folders["p"]), "--dtype", "float32",
+                           "--requests", str(tmp_path / "requests.json"), "--policy", "chunked", "--pages", "16",
+                           "--token-budget", "6", "--prefill-chunk", "3"], capture_output=True, text=True, timeout=300, env=env, cwd=str(tmp_path))
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    by_key = {r["key"]: r for r in json.loads(proc.stdout)["requests"]}
+    assert by_key["x"]["generated"] == P.greedy(cfg, w, [1, 2, 3, 4, 5, 6, 7], 5)
+    assert by_key["y"]["generated"] == P.greedy(cfg, w, [9], 4)
+    proc = subprocess.run([sys.executable, "-m", "runtime", "--model", "novosun-tiny", "--tokens", "5,6,7", "--max-new-tokens", "3",
+                           "--overlap", "--report"], capture_output=True, text=True, timeout=300, env=env, cwd=str(tmp_path))
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    out = json.loads(proc.stdout)
+    assert out["weights"] == "random-novosun-tiny" and len(out["requests"][0]["generated"]) == 3
+    assert out["runner"]["replays"] >= 1 and out["runner"]["cache"][0]["resident_pages"] == 0
