@@ -2,7 +2,7 @@
 engine's writer), and the plain implementation's logits for them.
 
 The configurations differ from each other in every size and constant, and inside each the sizes that could be
-confused are unequal: key and value sizes of a head, head counts of the two mixers of a layer, key/value heads,
+confused are unequal (one has no attention at all, so no pages): key and value sizes of a head, head counts of the two mixers of a layer, key/value heads,
 groups and norm groups, taps.  One has a width that is no multiple of 8, a single head and a convolution of one
 tap (no inputs to carry); one is drawn sharp: scores with a spread of several units, so that a query's result hangs
 on one key, often far back, and decays close to one, so that the state remembers the first tokens.
@@ -46,8 +46,10 @@ CONFIGS = {
         parallel((4, 1, 16, 32, 1.0), (2, 24, 16, 2, 3, 2), mlp(64, 2.0)),
         gla(2, 24, 16, 16.0, mlp(64, 2.0)),
         parallel((2, 1, 32, 16, 0.8), (3, 16, 8, 1, 5, 3))]),
+    # no layer keeps pages: the cache manager has state slots only
+    "g": config(53, 40, 0.6, 1e-5, [gla(2, 8, 12, 6.0, mlp(48, 2.0)), gla(1, 20, 8, 3.0)]),
 }
-SEEDS = {"p": 11, "q": 12, "s": 13}
+SEEDS = {"p": 11, "q": 12, "s": 13, "g": 14}
 
 
 def tensor_shapes(c, rank=6):

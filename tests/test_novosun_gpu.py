@@ -418,10 +418,10 @@ def test_far_keys_page_borders_and_old_state_in_a_model_drawn_sharp(folders, dty
     assert_close(got[:3], want[:3], dtype, "the first tokens")
 
 
-@pytest.mark.parametrize("dtype, execution, overlap", [("float32", "graph", True), ("float32", "eager", False), ("bfloat16", "graph", True)])
-def test_greedy_generation_through_the_scheduler(folders, dtype, execution, overlap):
+@pytest.mark.parametrize("name, dtype, execution, overlap", [("p", "float32", "graph", True), ("p", "float32", "eager", False),
+                                                             ("p", "bfloat16", "graph", True), ("g", "float32", "graph", True)])
+def test_greedy_generation_through_the_scheduler(folders, name, dtype, execution, overlap):
     from runtime.engine.scheduler import Engine
-    name = "p"
     cfg, w = P.read_folder(folders[name])
     prompts = [random_tokens(70 + i, n, cfg["vocab"]) for i, n in enumerate([11, 3, 26, 1, 40])]
     engine = Engine.from_folder(folders[name], dtype=dtype, pages=24, page_size=16, execution=execution,
