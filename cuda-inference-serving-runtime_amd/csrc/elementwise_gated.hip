@@ -132,7 +132,7 @@ extern "C" int cisr_glu_clamped(const void* gu, void* act, int rows, int inter, 
 }
 
 // ------------------------------------------------- per-head norm of queries and keys + scatter into the pages
-// One block a token row, a wave a head at a time.  The row of the fused projection is [q: heads x dim |
+// A wave a (token row, head); a block holds four heads of a row.  The row of the fused projection is [q: heads x dim |
 // k: kv_heads x dim | v: kv_heads x vdim | ...].  Queries go to q_out [T, heads, pad] (coordinates dim..pad-1 zero),
 // keys to kcache [pages, kv_heads, page_size, pad] (likewise), values transposed to vcache [pages, kv_heads, pad,
 // page_size] (coordinates vdim..pad-1 zero): heads of `pad` coordinates are what the attention kernels read.
@@ -147,7 +147,7 @@ qk_norm_scatter_kernel(const T* __restrict__ qkv, int ld, const float* __restric
     const T* src = qkv + (size_t)row * ld;
     const int slot = slots ? slots[row] : -1;
     const int items = heads + 2 * kv_heads;
-    for (int item = wave; item < items; item += 4) {
+    for (int item = blockIdx.y * 4 + wave; item < items; item += 4 * gridDim.y) {
         if (item < heads + kv_heads) {
             const bool is_q = item < heads;
             const int head = is_q ? item : item - heads;
@@ -186,11 +186,12 @@ extern "C" int cisr_qk_norm_scatter(const void* qkv, int ld, const float* wq, co
     if (dim <= 0 || vdim <= 0 || dim > pad || vdim > pad || pad > 256 || page_size <= 0 ||
         ld < (heads + kv_heads) * dim + kv_heads * vdim)
         return (int)hipErrorInvalidValue;
+    const dim3 grid(rows, min((heads + 2 * kv_heads + 3) / 4, 65535));
     if (dtype == DT_F32)
-        qk_norm_scatter_kernel<float><<<rows, 256, 0, stream>>>((const float*)qkv, ld, wq, wk, (float*)q_out, (float*)kcache,
+        qk_norm_scatter_kernel<float><<<grid, 256, 0, stream>>>((const float*)qkv, ld, wq, wk, (float*)q_out, (float*)kcache,
             (float*)vcache, slots, heads, kv_heads, dim, vdim, pad, page_size, eps);
     else
-        qk_norm_scatter_kernel<bf16_t><<<rows, 256, 0, stream>>>((const bf16_t*)qkv, ld, wq, wk, (bf16_t*)q_out, (bf16_t*)kcache,
+        qk_norm_scatter_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)qkv, ld, wq, wk, (bf16_t*)q_out, (bf16_t*)kcache,
             (bf16_t*)vcache, slots, heads, kv_heads, dim, vdim, pad, page_size, eps);
     return CISR_LAUNCH_CHECK();
 }
@@ -210,11 +211,37 @@ __global__ void head_gate_kernel(const T* __restrict__ attn, const T* __restrict
     store_f32(out + i, load_f32(attn + th * pad + d) * g);
 }
 
+// the same for bf16 with vdim and pad multiples of eight: eight elements a thread, 16-byte accesses
+__global__ void __launch_bounds__(256)
+head_gate_bf16x8_kernel(const bf16_t* __restrict__ attn, const bf16_t* __restrict__ gate, int ld_gate, bf16_t* __restrict__ out,
+                        int heads, int vdim8, int pad, size_t n8) {
+    typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n8) return;
+    const int d8 = (int)(i % vdim8);
+    const size_t th = i / vdim8;
+    const int h = (int)(th % heads);
+    const size_t t = th / heads;
+    const float g = gate ? 1.0f / (1.0f + expf(-bf16_to_f32(gate[t * ld_gate + h]))) : 1.0f;
+    const u32x4_t a = *(const u32x4_t*)(attn + th * pad + d8 * 8);
+    const uint32_t aw[4] = {a.x, a.y, a.z, a.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) o[k] = pack_bf16x2(__uint_as_float(aw[k] << 16) * g, __uint_as_float(aw[k] & 0xffff0000u) * g);
+    *(u32x4_t*)(out + i * 8) = (u32x4_t){o[0], o[1], o[2], o[3]};
+}
+
 extern "C" int cisr_head_gate(const void* attn, const void* gate, int ld_gate, void* out, int rows, int heads, int vdim,
                               int pad, int dtype, hipStream_t stream) {
     const size_t n = (size_t)rows * heads * vdim;
     if (n == 0) return 0;
     if (vdim > pad) return (int)hipErrorInvalidValue;
+    if (dtype == DT_BF16 && vdim % 8 == 0 && pad % 8 == 0 && ((uintptr_t)attn) % 16 == 0 && ((uintptr_t)out) % 16 == 0) {
+        const size_t n8 = n / 8;
+        head_gate_bf16x8_kernel<<<(unsigned)((n8 + 255) / 256), 256, 0, stream>>>((const bf16_t*)attn, (const bf16_t*)gate, ld_gate,
+                                                                                (bf16_t*)out, heads, vdim / 8, pad, n8);
+        return CISR_LAUNCH_CHECK();
+    }
     const unsigned blocks = (unsigned)((n + 255) / 256);
     if (dtype == DT_F32) head_gate_kernel<float><<<blocks, 256, 0, stream>>>((const float*)attn, (const float*)gate, ld_gate, (float*)out, heads, vdim, pad, n);
     else head_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)attn, (const bf16_t*)gate, ld_gate, (bf16_t*)out, heads, vdim, pad, n);

@@ -137,8 +137,9 @@ __global__ void decay_gate_kernel(const float* __restrict__ z, int ld, const flo
     a[i] = expf((fminf(u, 0.f) - log1pf(expf(-fabsf(u)))) * inv_tau);
 }
 
-// The same with z = up . low made on the way: z[t, c] = sum_r up[c * rank + r] * low[t * ld + r] (the second half of a
-// low-rank projection; the first half came out of the mixer's fused input product).
+// The same with z = up . low made on the way: z[t, c] = sum_r up_t[r * cols + c] * low[t * ld + r] (the second half of a
+// low-rank projection, its matrix transposed so that neighbouring lanes read neighbouring words; the first half came
+// out of the mixer's fused input product).
 __global__ void decay_gate_low_rank_kernel(const float* __restrict__ low, int ld, int rank, const float* __restrict__ up,
                                            const float* __restrict__ bias, float* __restrict__ a, int cols, size_t n, float inv_tau) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -146,9 +147,10 @@ __global__ void decay_gate_low_rank_kernel(const float* __restrict__ low, int ld
     const size_t t = i / cols;
     const int c = (int)(i % cols);
     const float* lo = low + t * ld;
-    const float* w = up + (size_t)c * rank;
+    const float* w = up + c;
     float u = bias ? bias[c] : 0.f;
-    for (int r = 0; r < rank; ++r) u += w[r] * lo[r];
+#pragma unroll 4
+    for (int r = 0; r < rank; ++r) u += w[(size_t)r * cols] * lo[r];
     a[i] = expf((fminf(u, 0.f) - log1pf(expf(-fabsf(u)))) * inv_tau);
 }
 

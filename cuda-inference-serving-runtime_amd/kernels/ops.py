@@ -1066,12 +1066,12 @@ def decay_gate(z, bias, out, tau):
 
 
 def decay_gate_low_rank(low, up, bias, out, tau):
-    """out = sigmoid(low . up^T + bias)^(1 / tau) in float: low a float view [T, rank] (the first half of a low-rank
-    projection), up float [N, rank], bias float [N] or None, out float [T, N]."""
+    """out = sigmoid(low . up + bias)^(1 / tau) in float: low a float view [T, rank] (the first half of a low-rank
+    projection), up float [rank, N] (the second half's matrix, transposed), bias float [N] or None, out float [T, N]."""
     T, rank = low.shape
-    n = up.shape[0]
+    n = up.shape[1]
     lp, ld = _rows_of(low, "low")
-    _check(_rec().cisr_decay_gate_low_rank(lp, ld, rank, _dev(up, "up", torch.float32, (n, rank)),
+    _check(_rec().cisr_decay_gate_low_rank(lp, ld, rank, _dev(up, "up", torch.float32, (rank, n)),
                                            None if bias is None else _dev(bias, "bias", torch.float32, (n,)),
                                            _dev(out, "out", torch.float32, (T, n)), T, n, float(tau), _stream()), "decay_gate_low_rank")
     return out

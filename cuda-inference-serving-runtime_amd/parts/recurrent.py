@@ -71,10 +71,10 @@ class GatedLinearAttention(Mixer):
         # few multiplications a decay, done in float by the kernel that makes the decays
         parts = [matrix_operand(tensors[self._tensor(p)], dtype) for p in ("q", "k", "v", "gate", "down")]
         self.low_rank = parts[-1].shape[0]
-        self.w_up = _float(tensors[self._tensor("up")])
-        if self.low_rank != self.w_up.shape[1]:
+        self.w_up = _float(tensors[self._tensor("up")].t())          # [rank, heads * dim]: the decays' kernel reads it by columns
+        if self.low_rank != self.w_up.shape[0]:
             raise ValueError(f"{self.name}: the decay's projections disagree about their inner size "
-                             f"({self.low_rank} and {self.w_up.shape[1]})")
+                             f"({self.low_rank} and {self.w_up.shape[0]})")
         self.w_in = torch.cat(parts, dim=0).contiguous()
         self.w_out = matrix_operand(tensors[self._tensor("o")], dtype)
         self.norm_weight, self.bias = _float(tensors[self._tensor("norm")]), _float(tensors[self._tensor("bias")])

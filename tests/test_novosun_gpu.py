@@ -176,7 +176,7 @@ def test_decay_gate_group_norm_gate_post_norm_and_clamped_gate():
     close(out.cpu().numpy(), P.sigmoid(z[:, 4:] + bias) ** (1 / 7.0))
     up = rng.standard_normal((9, 13))                     # the same with the second half of a low-rank projection on the way
     out = torch.zeros((T, 9), device=DEV)
-    ops.decay_gate_low_rank(full[:, 4:], dev(up), dev(bias[:9]), out, 3.0)
+    ops.decay_gate_low_rank(full[:, 4:], dev(up.T), dev(bias[:9]), out, 3.0)
     close(out.cpu().numpy(), P.sigmoid(z[:, 4:] @ up.T + bias[:9]) ** (1 / 3.0))
     # the norm of a mixer's result: gate after the norm with a weight shared by the heads; gate before it with a skip term
     heads, V = 3, 10
