@@ -57,11 +57,64 @@ post_norm_add_kernel(float* __restrict__ x, const float* __restrict__ a, const f
     for (int d = threadIdx.x; d < dim; d += 256) store_f32(out + d, (KEEP ? kept[d] : xr[d]) * rs * next_w[d]);
 }
 
+// The same for rows of up to 4,096 floats: a thread holds E elements of every operand in registers, so that all of a
+// row's loads are on their way together (one trip to memory instead of one a pass).
+template <bool TWO, int E, typename T>
+__global__ void __launch_bounds__(256)
+post_norm_add_short_kernel(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ wa,
+                           const float* __restrict__ b, const float* __restrict__ wb, const float* __restrict__ w,
+                           int dim, float eps, float mult, const float* __restrict__ next_w, float next_eps, T* __restrict__ next_out) {
+    __shared__ float red[4];
+    const size_t row = blockIdx.x;
+    float va[E], vb[E], vx[E], vw[E], vwa[E], vwb[E], vn[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        const int d = threadIdx.x + 256 * e;
+        const bool in = d < dim;
+        const int dd = in ? d : 0;
+        va[e] = in ? a[row * dim + dd] : 0.f;
+        vx[e] = in ? x[row * dim + dd] : 0.f;
+        vw[e] = w ? w[dd] : 1.f;
+        vn[e] = next_w ? next_w[dd] : 0.f;
+        if (TWO) { vb[e] = in ? b[row * dim + dd] : 0.f; vwa[e] = wa[dd]; vwb[e] = wb[dd]; }
+    }
+    float sa = 0.f, sb = 0.f;
+#pragma unroll
+    for (int e = 0; e < E; ++e) { sa += va[e] * va[e]; if (TWO) sb += vb[e] * vb[e]; }
+    if (TWO) {
+        const float ra = 0.5f / sqrtf(block_sum<256>(sa, red) / (float)dim + eps);
+        const float rb = 0.5f / sqrtf(block_sum<256>(sb, red) / (float)dim + eps);
+        sa = 0.f;
+#pragma unroll
+        for (int e = 0; e < E; ++e) { va[e] = va[e] * ra * vwa[e] + vb[e] * rb * vwb[e]; sa += va[e] * va[e]; }
+    }
+    const float scale = w ? mult / sqrtf(block_sum<256>(sa, red) / (float)dim + eps) : mult;
+    float sn = 0.f;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        const int d = threadIdx.x + 256 * e;
+        vx[e] += va[e] * scale * vw[e];
+        if (d < dim) { x[row * dim + d] = vx[e]; sn += vx[e] * vx[e]; }
+    }
+    if (next_w == nullptr) return;
+    const float rs = 1.0f / sqrtf(block_sum<256>(sn, red) / (float)dim + next_eps);
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        const int d = threadIdx.x + 256 * e;
+        if (d < dim) store_f32(next_out + row * dim + d, vx[e] * rs * vn[e]);
+    }
+}
+
 template <bool TWO, typename T>
 static void launch_post_norm_add(float* x, const float* a, const float* wa, const float* b, const float* wb, const float* w,
                                  int rows, int dim, float eps, float mult, const float* next_w, float next_eps, T* next_out,
                                  hipStream_t stream) {
-    if (dim <= 16384) post_norm_add_kernel<TWO, true, T><<<rows, 256, (size_t)dim * sizeof(float), stream>>>(x, a, wa, b, wb, w, dim, eps, mult, next_w, next_eps, next_out);
+#define SHORT(E) post_norm_add_short_kernel<TWO, E, T><<<rows, 256, 0, stream>>>(x, a, wa, b, wb, w, dim, eps, mult, next_w, next_eps, next_out)
+    if (dim <= 1024) SHORT(4);
+    else if (dim <= 2048) SHORT(8);
+    else if (dim <= 4096) SHORT(16);
+#undef SHORT
+    else if (dim <= 16384) post_norm_add_kernel<TWO, true, T><<<rows, 256, (size_t)dim * sizeof(float), stream>>>(x, a, wa, b, wb, w, dim, eps, mult, next_w, next_eps, next_out);
     else post_norm_add_kernel<TWO, false, T><<<rows, 256, 0, stream>>>(x, a, wa, b, wb, w, dim, eps, mult, next_w, next_eps, next_out);
 }
 

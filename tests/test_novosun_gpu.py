@@ -189,20 +189,28 @@ def test_decay_gate_group_norm_gate_post_norm_and_clamped_gate():
         ops.group_norm_gate(dev(y), dev(g), dev(w2), out, 2, 1e-3, gate_first=True, skip=(dev(d), dev(x)))
         u = (y + np.repeat(d, 5) * x) * P.silu(g)
         close(out.float().cpu().numpy(), P.rms(u.reshape(T, 2, 15), 1e-3).reshape(T, -1) * w2, tol)
-    # a sublayer's result into the residual stream, alone and as the mean of two normed results
-    H = 300
-    x0, a, b = rng.standard_normal((T, H)), rng.standard_normal((T, H)), 3 * rng.standard_normal((T, H))
-    wa, wb, wn = (1 + 0.1 * rng.standard_normal(H) for _ in range(3))
-    x = dev(x0)
-    ops.post_norm_add(x, dev(a), dev(wn), 1e-2, 0.3)
-    close(x.cpu().numpy(), x0 + 0.3 * P.rmsnorm(a, wn, 1e-2))
-    x = dev(x0)
-    ops.post_norm_add(x, dev(a), dev(wn), 1e-2, 0.6, second=(dev(b), dev(wa), dev(wb)))
-    mean = 0.5 * (P.rmsnorm(a, wa, 1e-2) + P.rmsnorm(b, wb, 1e-2))
-    close(x.cpu().numpy(), x0 + 0.6 * P.rmsnorm(mean, wn, 1e-2))
-    x = dev(x0)
-    ops.post_norm_add(x, dev(a), None, 0.0, 1.0, second=(dev(b), dev(wa), dev(wb)))
-    close(x.cpu().numpy(), x0 + 0.5 * (P.rmsnorm(a, wa, 0.0) + P.rmsnorm(b, wb, 0.0)))
+    # a sublayer's result into the residual stream, alone and as the mean of two normed results, with the norm that reads
+    # the stream next made on the way: rows in registers (up to 4,096 floats), waiting in LDS (up to 16,384), read again
+    for H in (300, 2048, 5000, 17000):
+        x0, a, b = rng.standard_normal((T, H)), rng.standard_normal((T, H)), 3 * rng.standard_normal((T, H))
+        wa, wb, wn = (1 + 0.1 * rng.standard_normal(H) for _ in range(3))
+        x = dev(x0)
+        ops.post_norm_add(x, dev(a), dev(wn), 1e-2, 0.3)
+        close(x.cpu().numpy(), x0 + 0.3 * P.rmsnorm(a, wn, 1e-2))
+        x = dev(x0)
+        ahead = torch.zeros((T, H), device=DEV)
+        ops.post_norm_add(x, dev(a), dev(wn), 1e-2, 0.6, second=(dev(b), dev(wa), dev(wb)), following=(dev(wb), 1e-4, ahead))
+        mean = 0.5 * (P.rmsnorm(a, wa, 1e-2) + P.rmsnorm(b, wb, 1e-2))
+        close(x.cpu().numpy(), x0 + 0.6 * P.rmsnorm(mean, wn, 1e-2))
+        close(ahead.cpu().numpy(), P.rmsnorm(x0 + 0.6 * P.rmsnorm(mean, wn, 1e-2), wb, 1e-4))
+        x = dev(x0)
+        ops.post_norm_add(x, dev(a), None, 0.0, 1.0, second=(dev(b), dev(wa), dev(wb)))
+        close(x.cpu().numpy(), x0 + 0.5 * (P.rmsnorm(a, wa, 0.0) + P.rmsnorm(b, wb, 0.0)))
+        x = dev(x0)
+        ahead = torch.zeros((T, H), device=DEV, dtype=torch.bfloat16)
+        ops.post_norm_add(x, dev(a), dev(wn), 1e-2, 0.3, following=(dev(wa), 1e-3, ahead))
+        close(x.cpu().numpy(), x0 + 0.3 * P.rmsnorm(a, wn, 1e-2))
+        close(ahead.float().cpu().numpy(), P.rmsnorm(x0 + 0.3 * P.rmsnorm(a, wn, 1e-2), wa, 1e-3), 8e-3)
     for inter in (21, 24):                                 # (rows of a multiple of eight: 16-byte accesses)
         gu = rng.standard_normal((T, 2 * inter)) * 3
         for dtype, tol in ((torch.float32, 2e-5), (torch.bfloat16, 8e-3)):
@@ -210,14 +218,6 @@ def test_decay_gate_group_norm_gate_post_norm_and_clamped_gate():
             out = ops.glu_clamped(operand, torch.zeros((T, inter), device=DEV, dtype=dtype), 1.25)
             ref = operand.float().cpu().numpy()
             close(out.float().cpu().numpy(), P.clamped_glu(ref[:, :inter], ref[:, inter:], 1.25), tol)
-    # the norm that reads the residual stream next, made on the way
-    x = dev(x0)
-    ahead = torch.zeros((T, H), device=DEV, dtype=torch.bfloat16)
-    ops.post_norm_add(x, dev(a), dev(wn), 1e-2, 0.3, following=(dev(wa), 1e-3, ahead))
-    close(x.cpu().numpy(), x0 + 0.3 * P.rmsnorm(a, wn, 1e-2))
-    close(ahead.float().cpu().numpy(), P.rmsnorm(x0 + 0.3 * P.rmsnorm(a, wn, 1e-2), wa, 1e-3), 8e-3)
-
-
 @pytest.mark.parametrize("rows", [1, 3, 16, 40, 100])
 @pytest.mark.parametrize("inner, width", [(64, 48), (1024, 4096)])
 def test_clamped_gate_as_the_epilogue_of_the_product_over_gate_and_up(rows, inner, width):
