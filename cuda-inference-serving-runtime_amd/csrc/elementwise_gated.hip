@@ -58,12 +58,14 @@ post_norm_add_kernel(float* __restrict__ x, const float* __restrict__ a, const f
 }
 
 // The same for rows of up to 4,096 floats: a thread holds E elements of every operand in registers, so that all of a
-// row's loads are on their way together (one trip to memory instead of one a pass).
+// row's loads are on their way together (one trip to memory instead of one a pass).  slices_a / slices_b > 0: a (b) is
+// a product that was cut along its inner size and left as partial sums [slices][rows][dim], added here in slice order.
 template <bool TWO, int E, typename T>
 __global__ void __launch_bounds__(256)
 post_norm_add_short_kernel(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ wa,
                            const float* __restrict__ b, const float* __restrict__ wb, const float* __restrict__ w,
-                           int dim, float eps, float mult, const float* __restrict__ next_w, float next_eps, T* __restrict__ next_out) {
+                           int dim, float eps, float mult, const float* __restrict__ next_w, float next_eps, T* __restrict__ next_out,
+                           int slices_a, int slices_b) {
     __shared__ float red[4];
     const size_t row = blockIdx.x;
     float va[E], vb[E], vx[E], vw[E], vwa[E], vwb[E], vn[E];
@@ -78,6 +80,25 @@ post_norm_add_short_kernel(float* __restrict__ x, const float* __restrict__ a, c
         vn[e] = next_w ? next_w[dd] : 0.f;
         if (TWO) { vb[e] = in ? b[row * dim + dd] : 0.f; vwa[e] = wa[dd]; vwb[e] = wb[dd]; }
     }
+    // the further slices of a cut product, four slices' loads on their way at a time, added in slice order
+    auto add_slices = [&](float (&v)[E], const float* parts, int slices) {
+        for (int s0 = 1; s0 < slices; s0 += 4) {
+            float more[4][E];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    const int d = threadIdx.x + 256 * e;
+                    more[j][e] = (s0 + j < slices && d < dim) ? parts[((size_t)(s0 + j) * gridDim.x + row) * dim + d] : 0.f;
+                }
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int e = 0; e < E; ++e) v[e] += more[j][e];
+        }
+    };
+    if (slices_a > 1) add_slices(va, a, slices_a);
+    if (TWO && slices_b > 1) add_slices(vb, b, slices_b);
     float sa = 0.f, sb = 0.f;
 #pragma unroll
     for (int e = 0; e < E; ++e) { sa += va[e] * va[e]; if (TWO) sb += vb[e] * vb[e]; }
@@ -108,8 +129,8 @@ post_norm_add_short_kernel(float* __restrict__ x, const float* __restrict__ a, c
 template <bool TWO, typename T>
 static void launch_post_norm_add(float* x, const float* a, const float* wa, const float* b, const float* wb, const float* w,
                                  int rows, int dim, float eps, float mult, const float* next_w, float next_eps, T* next_out,
-                                 hipStream_t stream) {
-#define SHORT(E) post_norm_add_short_kernel<TWO, E, T><<<rows, 256, 0, stream>>>(x, a, wa, b, wb, w, dim, eps, mult, next_w, next_eps, next_out)
+                                 int slices_a, int slices_b, hipStream_t stream) {
+#define SHORT(E) post_norm_add_short_kernel<TWO, E, T><<<rows, 256, 0, stream>>>(x, a, wa, b, wb, w, dim, eps, mult, next_w, next_eps, next_out, slices_a, slices_b)
     if (dim <= 1024) SHORT(4);
     else if (dim <= 2048) SHORT(8);
     else if (dim <= 4096) SHORT(16);
@@ -120,16 +141,17 @@ static void launch_post_norm_add(float* x, const float* a, const float* wa, cons
 
 extern "C" int cisr_post_norm_add(float* x, const float* a, const float* wa, const float* b, const float* wb,
                                   const float* w, int rows, int dim, float eps, float mult, const float* next_w, float next_eps,
-                                  void* next_out, int next_dtype, hipStream_t stream) {
+                                  void* next_out, int next_dtype, int slices_a, int slices_b, hipStream_t stream) {
     if (rows <= 0) return 0;
-    if (dim <= 0 || (b != nullptr && (wa == nullptr || wb == nullptr)) || (next_w != nullptr && next_out == nullptr))
+    if (dim <= 0 || (b != nullptr && (wa == nullptr || wb == nullptr)) || (next_w != nullptr && next_out == nullptr) ||
+        slices_a < 0 || slices_b < 0 || ((slices_a > 0 || slices_b > 0) && dim > 4096))    // (partial sums: the kernel of short rows)
         return (int)hipErrorInvalidValue;
     if (next_dtype == DT_F32) {
-        if (b) launch_post_norm_add<true, float>(x, a, wa, b, wb, w, rows, dim, eps, mult, next_w, next_eps, (float*)next_out, stream);
-        else launch_post_norm_add<false, float>(x, a, nullptr, nullptr, nullptr, w, rows, dim, eps, mult, next_w, next_eps, (float*)next_out, stream);
+        if (b) launch_post_norm_add<true, float>(x, a, wa, b, wb, w, rows, dim, eps, mult, next_w, next_eps, (float*)next_out, slices_a, slices_b, stream);
+        else launch_post_norm_add<false, float>(x, a, nullptr, nullptr, nullptr, w, rows, dim, eps, mult, next_w, next_eps, (float*)next_out, slices_a, slices_b, stream);
     } else {
-        if (b) launch_post_norm_add<true, bf16_t>(x, a, wa, b, wb, w, rows, dim, eps, mult, next_w, next_eps, (bf16_t*)next_out, stream);
-        else launch_post_norm_add<false, bf16_t>(x, a, nullptr, nullptr, nullptr, w, rows, dim, eps, mult, next_w, next_eps, (bf16_t*)next_out, stream);
+        if (b) launch_post_norm_add<true, bf16_t>(x, a, wa, b, wb, w, rows, dim, eps, mult, next_w, next_eps, (bf16_t*)next_out, slices_a, slices_b, stream);
+        else launch_post_norm_add<false, bf16_t>(x, a, nullptr, nullptr, nullptr, w, rows, dim, eps, mult, next_w, next_eps, (bf16_t*)next_out, slices_a, slices_b, stream);
     }
     return CISR_LAUNCH_CHECK();
 }

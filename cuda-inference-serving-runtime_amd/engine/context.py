@@ -105,6 +105,14 @@ class StepContext:
                 return residual
         return ops.gemm(a, w, residual, residual=residual, scratch=self.scratch)
 
+    def product_for_norm(self, a, w, tag):
+        """a . w^T as float rows [T, N] in the buffer `tag`, for a part whose result is read next by the kernel that adds
+        it to the residual stream (ops.post_norm_add): where the wide kernel cuts the product, its partial sums are left
+        to that kernel (an ops.Partials in a buffer of its own, `tag`.parts) instead of a finishing kernel here."""
+        rows, cols = a.shape[0], w.shape[0]
+        return ops.gemm_for_norm(a, w, self.buffer(tag, (rows, cols), torch.float32),
+                                 lambda floats: self.buffer(tag + ".parts", (floats,), torch.float32), scratch=self.scratch)
+
     def leave_unfinished(self, rows, partials):
         """`rows` lack the partial sums `partials` (ops.gemm_unfinished); whoever reads them next adds them."""
         if self.unfinished is not None:

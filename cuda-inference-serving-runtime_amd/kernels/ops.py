@@ -69,7 +69,7 @@ def _declare(h):
         "cisr_gemm_skinny_bf16_gated": [p, i, p, i, p, i, i, i, i, i, f, f, f, p],
         "cisr_gemm_wide_bf16_gated": [p, i, p, i, p, i, i, i, i, i, f, f, f, p, C.c_longlong, p],
         "cisr_gemm_bf16_gated": [p, i, p, i, p, i, i, i, i, i, f, f, f, p],
-        "cisr_post_norm_add": [p, p, p, p, p, p, i, i, f, f, p, f, p, i, p],
+        "cisr_post_norm_add": [p, p, p, p, p, p, i, i, f, f, p, f, p, i, i, i, p],
         "cisr_glu_clamped": [p, p, i, i, f, f, f, i, p],
         "cisr_qk_norm_scatter": [p, i, p, p, p, p, p, p, i, i, i, i, i, i, i, f, i, p],
         "cisr_head_gate": [p, p, i, p, i, i, i, i, i, p],
@@ -852,26 +852,64 @@ def take_tokens(tokens, source, sampled):
 
 # -- layers that norm a sublayer's output, clamped gates, normed and gated attention ----------------------------------
 
+class Partials:
+    """A product [rows, cols] that the wide kernel cut along its inner size and left as partial sums: `parts` float
+    [slices * rows * cols], to be added in slice order by the kernel that reads the product next (post_norm_add)."""
+
+    def __init__(self, parts, slices, rows, cols):
+        self.parts, self.slices, self.rows, self.cols = parts, int(slices), int(rows), int(cols)
+
+
+PARTIALS_MAX_COLS = 4096      # rows that post_norm_add holds in registers: only those take partial sums
+
+
+def gemm_for_norm(a, w, out, make_buffer, scratch=None):
+    """a . w^T for a reader that can add partial sums (post_norm_add): where the wide kernel cuts the product along
+    its inner size, its slices' partial sums are left in a buffer of the caller's (`make_buffer(floats)`: not the
+    shared scratch, which the next wide product would overwrite) and a Partials is returned; every other product is
+    finished into `out` (float [M, N]) and `out` is returned."""
+    m, k = a.shape
+    n = w.shape[0]
+    if (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and 0 < m <= SKINNY_ROWS and n <= PARTIALS_MAX_COLS
+            and not library_ok(m, w) and _skinny_ok(a, w) and wide_ok(m, w)):
+        need = _wide_plan(m, n, k, False)
+        if need > 0:
+            work = make_buffer(need)
+            _check(lib().cisr_gemm_wide_partials_bf16(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), m, n, k,
+                                                      _dev(work, "partial sums", torch.float32), work.numel(), _stream()), "gemm_for_norm")
+            return Partials(work, need // (m * n), m, n)
+    return gemm(a, w, out, scratch=scratch)
+
+
 def post_norm_add(x, y, weight, eps, mult, second=None, following=None):
     """x += mult * rmsnorm(y) * weight, in place (all float, [T, H]).  With `second` = (y2, w1, w2) the row that is
     normed is (rmsnorm(y) w1 + rmsnorm(y2) w2) / 2: two sublayers side by side.  `weight` None: no outer norm,
     x += mult * row.  `following` = (weight float [H], eps, out [T, H] float or bf16): the norm that reads x next is made
-    by the same kernel, out = rmsnorm(x) * weight."""
+    by the same kernel, out = rmsnorm(x) * weight.  y (and y2) may be a Partials of [T, H]: its slices are added on the way."""
     rows, dim = x.shape
     xp = _dev(x, "x", torch.float32)
-    yp = _dev(y, "y", torch.float32, (rows, dim))
+
+    def operand(t, name):
+        if isinstance(t, Partials):
+            if (t.rows, t.cols) != (rows, dim) or dim > PARTIALS_MAX_COLS or t.parts.numel() < t.slices * rows * dim:
+                raise KernelError(f"post_norm_add: {name} is not the partial sums of a product [{rows}, {dim}]")
+            return _dev(t.parts, name, torch.float32), t.slices
+        return _dev(t, name, torch.float32, (rows, dim)), 0
+
+    yp, slices_a = operand(y, "y")
+    slices_b = 0
     wp = None if weight is None else _dev(weight, "weight", torch.float32, (dim,))
     ap = bp = w2p = None
     if second is not None:
         y2, w1, w2 = second
-        bp = _dev(y2, "y2", torch.float32, (rows, dim))
+        bp, slices_b = operand(y2, "y2")
         ap, w2p = _dev(w1, "w1", torch.float32, (dim,)), _dev(w2, "w2", torch.float32, (dim,))
     np_, neps, op, odt = None, 0.0, None, F32
     if following is not None:
         nw, neps, out = following
         np_, op, odt = _dev(nw, "following weight", torch.float32, (dim,)), _dev(out, "following out", None, (rows, dim)), _storage(out, "following out")
     _check(lib().cisr_post_norm_add(xp, yp, ap, bp, w2p, wp, rows, dim, float(eps), float(mult), np_, float(neps), op, odt,
-                                    _stream()), "post_norm_add")
+                                    slices_a, slices_b, _stream()), "post_norm_add")
     return x
 
 

@@ -201,10 +201,11 @@ class NormedGatedAttention(Mixer):
         first_gate = (nh + nkv) * D + nkv * V
         gates = qkv[:, first_gate:first_gate + nh] if self.head_gate else None
         act = ops.head_gate(out, gates, ctx.buffer("gattn.act", (T, nh * V), ctx.dtype), nh, V, pad)
-        return ops.gemm(act, self.w_out, ctx.buffer("gattn.y", (T, self.hidden), torch.float32), scratch=ctx.scratch)
+        return ctx.product_for_norm(act, self.w_out, "gattn.y")
 
     def forward(self, h, residual, ctx, site, norm=None):
-        return ops.residual_add(residual, self.output(h, ctx, site))
+        from .block import add_sublayer
+        return add_sublayer(residual, self.output(h, ctx, site), None, 1.0)
 
 
 register_part("mixer", "attention", PagedAttention)

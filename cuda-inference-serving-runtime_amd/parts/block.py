@@ -70,7 +70,7 @@ class PreNormBlock(Part):
 
 class NormedMean:
     """What a mixer made of two mixers side by side hands to the arrangement around it: half the sum of two results,
-    each RMS-normed over the width with a weight of its own (float [T, H] each).  The arrangement's kernel that adds
+    each RMS-normed over the width with a weight of its own (float [T, H] each, or the partial sums of a cut product).  The arrangement's kernel that adds
     a sublayer's result to the residual stream makes the mean on the way (ops.post_norm_add)."""
 
     def __init__(self, first, first_weight, second, second_weight, eps):

@@ -85,10 +85,11 @@ class ClampedGLU(FeedForward):
         else:
             ops.gemm_swiglu(h, self.w_gate_up, act, gate_up=ctx.buffer("ffn.gate_up", (T, 2 * self.intermediate), ctx.dtype),
                             scratch=ctx.scratch, law=law)
-        return ops.gemm(act, self.w_down, ctx.buffer("ffn.out", (T, self.hidden), torch.float32), scratch=ctx.scratch)
+        return ctx.product_for_norm(act, self.w_down, "ffn.out")
 
     def forward(self, h, residual, ctx, norm=None):
-        return ops.residual_add(residual, self.output(h, ctx))
+        from .block import add_sublayer
+        return add_sublayer(residual, self.output(h, ctx), None, 1.0)
 
 
 register_part("ffn", "gated_mlp", GatedMLP)

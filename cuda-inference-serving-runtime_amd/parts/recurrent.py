@@ -90,10 +90,11 @@ class GatedLinearAttention(Mixer):
               self.heads, self.dim, self.vdim, q_scale=self.dim ** -0.5)
         act = ops.group_norm_gate(o, proj[:, 2 * K + V:2 * K + 2 * V], self.norm_weight, ctx.buffer("gla.act", (T, V), ctx.dtype),
                                   self.heads, self.eps, gate_first=False, shared_weight=True)
-        return ops.gemm(act, self.w_out, ctx.buffer("gla.y", (T, self.hidden), torch.float32), scratch=ctx.scratch)
+        return ctx.product_for_norm(act, self.w_out, "gla.y")
 
     def forward(self, h, residual, ctx, site, norm=None):
-        return ops.residual_add(residual, self.output(h, ctx, site))
+        from .block import add_sublayer
+        return add_sublayer(residual, self.output(h, ctx, site), None, 1.0)
 
 
 class StateSpaceDuality(Mixer):
@@ -154,10 +155,11 @@ class StateSpaceDuality(Mixer):
               nh, self.state, self.vdim, share=nh // self.groups, step=step)
         act = ops.group_norm_gate(y, proj[:, :inner], self.norm_weight, ctx.buffer("ssd.act", (T, inner), ctx.dtype),
                                   self.norm_groups, self.eps, gate_first=True, skip=(self.skip, xbc[:, :inner]))
-        return ops.gemm(act, self.w_out, ctx.buffer("ssd.y", (T, self.hidden), torch.float32), scratch=ctx.scratch)
+        return ctx.product_for_norm(act, self.w_out, "ssd.y")
 
     def forward(self, h, residual, ctx, site, norm=None):
-        return ops.residual_add(residual, self.output(h, ctx, site))
+        from .block import add_sublayer
+        return add_sublayer(residual, self.output(h, ctx, site), None, 1.0)
 
 
 class SideBySide(Mixer):

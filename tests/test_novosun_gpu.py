@@ -218,6 +218,42 @@ def test_decay_gate_group_norm_gate_post_norm_and_clamped_gate():
             out = ops.glu_clamped(operand, torch.zeros((T, inter), device=DEV, dtype=dtype), 1.25)
             ref = operand.float().cpu().numpy()
             close(out.float().cpu().numpy(), P.clamped_glu(ref[:, :inter], ref[:, inter:], 1.25), tol)
+@pytest.mark.parametrize("rows", [1, 8, 24, 64])
+def test_a_cut_product_is_left_to_the_sum_that_reads_it(rows):
+    """Against large weights the wide kernel cuts a product along its inner size; the kernel that adds a sublayer's
+    result to the residual stream takes the slices' partial sums instead of a finished product (alone, and as both
+    halves of a mean of two results)."""
+    from runtime.kernels import ops
+    rng = np.random.default_rng(rows)
+    K, N = 8192, 2048
+    a1, a2 = (dev(rng.standard_normal((rows, K)), torch.bfloat16) for _ in range(2))
+    w1, w2 = (dev(rng.standard_normal((N, K)) / np.sqrt(K), torch.bfloat16) for _ in range(2))
+    made = []
+
+    def product(a, w):
+        kept = {}
+        got = ops.gemm_for_norm(a, w, torch.zeros((rows, N), device=DEV), lambda n: kept.setdefault("parts", torch.zeros(n, device=DEV)))
+        made.append(isinstance(got, ops.Partials))
+        return got
+
+    y1, y2 = product(a1, w1), product(a2, w2)
+    if rows > 4:
+        assert all(made) and y1.slices >= 2, "this shape was meant to be cut"
+    r1, r2 = (a.float() @ w.float().T for a, w in ((a1, w1), (a2, w2)))
+    x0 = rng.standard_normal((rows, N))
+    wn, wa, wb = (1 + 0.1 * rng.standard_normal(N) for _ in range(3))
+    x = dev(x0)
+    ahead = torch.zeros((rows, N), device=DEV)
+    ops.post_norm_add(x, y1, dev(wn), 1e-5, 0.3, following=(dev(wa), 1e-5, ahead))
+    want = x0 + 0.3 * P.rmsnorm(r1.cpu().numpy(), wn, 1e-5)
+    close(x.cpu().numpy(), want, 1e-4)
+    close(ahead.cpu().numpy(), P.rmsnorm(want, wa, 1e-5), 1e-4)
+    x = dev(x0)
+    ops.post_norm_add(x, y1, dev(wn), 1e-5, 0.5, second=(y2, dev(wa), dev(wb)))
+    mean = 0.5 * (P.rmsnorm(r1.cpu().numpy(), wa, 1e-5) + P.rmsnorm(r2.cpu().numpy(), wb, 1e-5))
+    close(x.cpu().numpy(), x0 + 0.5 * P.rmsnorm(mean, wn, 1e-5), 1e-4)
+
+
 @pytest.mark.parametrize("rows", [1, 3, 16, 40, 100])
 @pytest.mark.parametrize("inner, width", [(64, 48), (1024, 4096)])
 def test_clamped_gate_as_the_epilogue_of_the_product_over_gate_and_up(rows, inner, width):
