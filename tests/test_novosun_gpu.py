@@ -362,6 +362,34 @@ def test_prompt_then_tokens_one_by_one_and_portions_down_to_two_tokens(folders, 
     runner.cache.check()
 
 
+@pytest.mark.parametrize("name, dtype, execution", [("q", "float32", "graph"), ("p", "bfloat16", "graph"), ("s", "float32", "eager")])
+def test_long_decoding_from_the_first_token(folders, name, dtype, execution):
+    """A request decoded one token at a time from its very first token, over a dozen pages, beside a second request that
+    joins late and leaves early (its slot and pages go back while the first goes on)."""
+    from runtime.engine import StepEntry
+    V = CONFIGS[name]["vocab"]
+    long, short = random_tokens(21, 210, V), random_tokens(22, 40, V)
+    want = {"l": plain_logits(folders[name], long), "s": plain_logits(folders[name], short)}
+    runner = make_runner(folders[name], dtype, pages=17, execution=execution)
+    runner.create("l")
+    got = {"l": [], "s": []}
+    for t, token in enumerate(long):
+        entries = [StepEntry("l", [token], [0])]
+        if 60 <= t < 100:
+            if t == 60:
+                runner.create("s")
+            entries.append(StepEntry("s", [short[t - 60]], [0]))
+        out = runner.step(entries).cpu().numpy()
+        got["l"].append(out[0])
+        if len(entries) == 2:
+            got["s"].append(out[1])
+        if t == 99:
+            runner.release("s")
+    assert_close(np.stack(got["l"]), want["l"], dtype, "long decoding")
+    assert_close(np.stack(got["s"]), want["s"], dtype, "the request that joined late")
+    runner.cache.check()
+
+
 def mixed(V, seed, lengths=(70, 33, 120, 9, 64, 97, 40, 130), live_at_once=4):
     """Up to `live_at_once` live requests: portions of some beside single tokens of others; requests end and new ones
     start on the pages and state slots they gave back; one request sits out some steps."""
