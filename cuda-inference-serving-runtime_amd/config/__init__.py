@@ -2,4 +2,5 @@ from .base import (ConfigError, Architecture, register_architecture, unregister_
                    registered_architectures, architecture_of, read_config_json, config_from_folder)
 from .llama import LlamaConfig
 from .novosun import NovosunConfig
+from .ditazen import DitazenConfig
 from .presets import preset, preset_names

@@ -73,6 +73,11 @@ def _declare(h):
         "cisr_glu_clamped": [p, p, i, i, f, f, f, i, p],
         "cisr_qk_norm_scatter": [p, i, p, p, p, p, p, p, i, i, i, i, i, i, i, f, i, p],
         "cisr_head_gate": [p, p, i, p, i, i, i, i, i, p],
+        "cisr_layernorm": [p, p, p, p, p, i, i, f, i, p],
+        "cisr_rms_slice": [p, i, i, p, p, i, i, f, i, p],
+        "cisr_latent_keys": [p, i, i, p, p, i, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, i, i, f, i, p],
+        "cisr_heads_product": [p, i, i, p, p, i, i, p, i, i, i, i, i, i, p],
+        "cisr_gelu": [p, p, ll, i, i, p],
     }
     for name, args in sig.items():
         fn = getattr(h, name)
@@ -958,6 +963,92 @@ def head_gate(attn, gates, out, heads, vdim, pad):
     return out
 
 
+# -- layers with a centred norm, latent attention, an ungated feed-forward (csrc/elementwise_latent.hip) --------------
+
+def layernorm(x, weight, out, eps, rows=None, bias=None):
+    """out = (x[rows] - mean) / sqrt(var + eps) * weight (+ bias), var the mean of the squared deviations.
+    x float [T, H]; weight, bias float [H]; out [R, H] float or bf16."""
+    dim = x.shape[1]
+    n_out = out.shape[0]
+    if rows is None and n_out != x.shape[0]:
+        raise KernelError("layernorm: out rows differ from input rows")
+    rp = None if rows is None else _dev(rows, "rows", torch.int32, (n_out,))
+    bp = None if bias is None else _dev(bias, "bias", torch.float32, (dim,))
+    _check(lib().cisr_layernorm(_dev(x, "x", torch.float32), _dev(weight, "weight", torch.float32, (dim,)), bp,
+                                _dev(out, "out", None, (n_out, dim)), rp, n_out, dim, float(eps), _storage(out, "out"),
+                                _stream()), "layernorm")
+    return out
+
+
+def rms_slice(x, weight, out, eps):
+    """out = x / sqrt(mean(x^2) + eps) * weight over the columns of the float view x [T, n] of a row-major buffer;
+    weight float [n]; out [T, n] float or bf16."""
+    rows, n = x.shape
+    xp, ld = _rows_of(x, "x")
+    _check(lib().cisr_rms_slice(xp, ld, 0, _dev(weight, "weight", torch.float32, (n,)), _dev(out, "out", None, (rows, n)),
+                                rows, n, float(eps), _storage(out, "out"), _stream()), "rms_slice")
+    return out
+
+
+def latent_keys(down, weight, q, q_out, kcache, vcache, positions, slots, cos, sin, heads, dim, rot_dim, rank, pad,
+                page_size, eps, interleaved=False):
+    """Rows of a latent attention's down-projection `down` (a float view [T, rank + rot_dim]): the first `rank` columns
+    RMS-normed with `weight` are the latent c, the last `rot_dim` the key part that turns with the position (its first
+    2 * cos.shape[1] coordinates; pair i is (i, i + pairs) or, `interleaved`, (2i, 2i + 1)).  Written at `slots` as one
+    key head [c | turned | 0] of `pad` coordinates (kcache [pages, 1, page_size, pad]) and one value head [c | 0]
+    (vcache [pages, 1, pad, page_size]).  q [T, heads * (dim + rot_dim)]: the last rot_dim coordinates of each head are
+    turned alike and written to q_out[t, h, rank : rank + rot_dim], zeros behind them; q_out[t, h, :rank] is left to
+    the caller (the query's product with the key up-projection)."""
+    rows = q_out.shape[0]
+    dp, ld = _rows_of(down, "down", rank + rot_dim)
+    max_pos, half = cos.shape
+    if rank + rot_dim > pad or 2 * half > rot_dim or half <= 0:
+        raise KernelError(f"latent_keys: {rank} + {rot_dim} coordinates do not fit heads of {pad}, or {2 * half} turn among {rot_dim}")
+    if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] != heads * (dim + rot_dim) or q.shape[0] != rows or q.dtype != q_out.dtype:
+        raise KernelError("latent_keys: q must be [T, heads * (dim + rot_dim)] of the cache's dtype")
+    pages = kcache.shape[0]
+    sp = None if slots is None else _dev(slots, "slots", torch.int32, (rows,))
+    _check(lib().cisr_latent_keys(dp, ld, 0, _dev(weight, "weight", torch.float32, (rank,)), q.data_ptr(), q.stride(0),
+                                  _dev(q_out, "q_out", None, (rows, heads * pad)),
+                                  _dev(kcache, "kcache", q_out.dtype, (pages, 1, page_size, pad)),
+                                  _dev(vcache, "vcache", q_out.dtype, (pages, 1, pad, page_size)),
+                                  _dev(positions, "positions", torch.int32, (rows,)), sp,
+                                  _dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32, (max_pos, half)),
+                                  rows, heads, dim, rot_dim, 2 * half, rank, pad, page_size, max_pos, int(bool(interleaved)),
+                                  float(eps), _storage(q_out, "q_out"), _stream()), "latent_keys")
+    return q_out
+
+
+def heads_product(a, a_head, w, out, out_head, gate=None):
+    """out[t, h * out_head + n] = sum_k a[t, h * a_head + k] w[h, n, k], times sigmoid(gate[t, h]) if `gate` (a float view
+    [T, heads]) is given: a small matrix of its own for every head.  a, out row-major views of the compute dtype with
+    unit column stride; w [heads, N, K] contiguous."""
+    heads, n, k = w.shape
+    rows = a.shape[0]
+    if a.dtype != w.dtype or out.dtype != w.dtype or a.stride(1) != 1 or out.stride(1) != 1 or out.shape[0] != rows:
+        raise KernelError("heads_product: operands of one dtype with contiguous rows")
+    if a.shape[1] < (heads - 1) * a_head + k or out.shape[1] < (heads - 1) * out_head + n:
+        raise KernelError("heads_product: rows too short for their heads")
+    gp, ldg = (None, 0) if gate is None else _rows_of(gate, "gate", heads)
+    if gate is not None and gate.shape[0] != rows:
+        raise KernelError("heads_product: gates differ in rows")
+    _check(lib().cisr_heads_product(a.data_ptr(), a.stride(0), int(a_head), _dev(w, "w"), out.data_ptr(), out.stride(0),
+                                    int(out_head), gp, ldg, rows, heads, n, k, _storage(w, "w"), _stream()), "heads_product")
+    return out
+
+
+GELU_KINDS = {"gelu": 0, "gelu_erf": 0, "gelu_tanh": 1}
+
+
+def gelu(x, out, kind="gelu"):
+    """out = gelu(x): "gelu" the exact form with the error function, "gelu_tanh" the tanh form."""
+    if kind not in GELU_KINDS:
+        raise KernelError(f"gelu: unknown form {kind!r}")
+    _check(lib().cisr_gelu(_dev(x, "x"), _dev(out, "out", x.dtype, x.shape), x.numel(), GELU_KINDS[kind], _storage(x, "x"),
+                           _stream()), "gelu")
+    return out
+
+
 # -- mixers with a state per request (the kernels of csrc/recurrence.hip, a shared object of their own) ---------------
 
 _recurrence = None
@@ -974,6 +1065,8 @@ def _rec():
             "cisr_decay_gate": [p, i, p, p, i, i, f, p],
             "cisr_decay_gate_low_rank": [p, i, i, p, p, p, i, i, f, p],
             "cisr_group_norm_gate": [p, p, i, p, i, p, i, p, i, p, i, i, i, f, i, i, p],
+            "cisr_delta_scan": [p, i, p, i, p, i, p, i, p, i, p, i, p, ll, p, p, i, i, i, i, i, f, i, p],
+            "cisr_unit_heads": [p, i, i, i, i, i, f, f, p],
         }
         for name, args in sig.items():
             fn = getattr(h, name)
@@ -1136,4 +1229,42 @@ def group_norm_gate(y, gate, weight, out, groups, eps, gate_first, shared_weight
     _check(_rec().cisr_group_norm_gate(_dev(y, "y", torch.float32), gp, ldg, wp, int(shared_weight), dp, span, xp, ldx,
                                        _dev(out, "out", None, (T, width)), T, groups, size, float(eps), int(bool(gate_first)),
                                        _storage(out, "out"), _stream()), "group_norm_gate")
+    return out
+
+
+def unit_heads(x, heads, dim, scale=1.0, eps=1e-6):
+    """The float view x [T, heads * dim] in place: every head becomes x / sqrt(sum(x^2) + eps) * scale."""
+    xp, ld = _rows_of(x, "x", heads * dim)
+    _check(_rec().cisr_unit_heads(xp, ld, 0, x.shape[0], heads, dim, float(eps), float(scale), _stream()), "unit_heads")
+    return x
+
+
+def delta_scan(q, k, v, decay, write, out, state, seg_start, state_slots, heads, rows_of_state, cols_of_state, share=1,
+               q_scale=1.0, columns=None):
+    """Per segment and head, over the segment's rows in order: S <- g S; u = sigmoid(b) (v - S^T k); S <- S + k u^T;
+    o = q_scale S^T q, S [rows_of_state, cols_of_state] read from and written back to the segment's state slot.
+    q, k float views [T, heads / share * R]; v, out [T, heads * C]; decay (g) and write (b) [T, heads]; state float
+    [slots, >= heads * R * C]; seg_start int32 [S + 1]; state_slots int32 [S]."""
+    R, Cc = int(rows_of_state), int(cols_of_state)
+    T = v.shape[0]
+    segments = state_slots.shape[0]
+    if heads % share or R > 256:
+        raise KernelError("delta_scan: heads must divide into their groups and a state has at most 256 rows")
+    qp, ldq = _rows_of(q, "q", heads // share * R)
+    kp, ldk = _rows_of(k, "k", heads // share * R)
+    vp, ldv = _rows_of(v, "v", heads * Cc)
+    op, ldo = _rows_of(out, "out", heads * Cc)
+    gp, ldg = _rows_of(decay, "decay", heads)
+    bp, ldb = _rows_of(write, "write", heads)
+    if any(t.shape[0] != T for t in (q, k, decay, write, out)):
+        raise KernelError("delta_scan: operands differ in rows")
+    if state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < heads * R * Cc or not state.is_cuda:
+        raise KernelError("delta_scan: the state must be float [slots, >= heads * R * C]")
+    cols = int(columns or scan_columns(segments, heads, Cc))
+    while columns is None and cols > 4 and -(-R // (128 // cols)) > 16:
+        cols //= 2
+    _check(_rec().cisr_delta_scan(qp, ldq, kp, ldk, vp, ldv, gp, ldg, bp, ldb, op, ldo, state.data_ptr(), state.stride(0),
+                                  _dev(seg_start, "seg_start", torch.int32, (segments + 1,)),
+                                  _dev(state_slots, "state_slots", torch.int32, (segments,)), segments, heads, R, Cc,
+                                  int(share), float(q_scale), cols, _stream()), "delta_scan")
     return out

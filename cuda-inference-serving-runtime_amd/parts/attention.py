@@ -208,5 +208,115 @@ class NormedGatedAttention(Mixer):
         return add_sublayer(residual, self.output(h, ctx, site), None, 1.0)
 
 
+class LatentAttention(Mixer):
+    """Softmax attention whose keys and values are made from one latent a token (multi-head latent attention).
+
+    Per token the cache holds c = rms(Wdkv h)[:rank] * w (the latent) and kr = rot(Wdkv h [rank:]) (a key part that
+    turns with the position, shared by all heads).  Head j's key is [Wuk_j c | kr], its value Wuv_j c, its query
+    [q_j | rot(qr_j)] with `dim` plain and `rot_dim` turning coordinates; score = (q_j . Wuk_j c + rot(qr_j) . kr) scale,
+    softmax over the visible keys (all earlier ones, or the last `window`).  Queries come from one projection, or with
+    `q_rank` through a normed latent of their own: q = Wuq (rms(Wdq h) wq).  With `head_gate` a head's result is
+    multiplied by sigmoid((Wg h)_j).  Then the output projection.
+
+    The keys' up-projection is moved to the query's side: q'_j = Wuk_j^T q_j has `rank` coordinates, and the attention
+    is that of `heads` query heads [q'_j | rot(qr_j)] over ONE key head [c | kr] and one value head [c] of
+    pad = rank + rot_dim coordinates (rounded up to 8, the rest zero), which the framework's paged attention kernels
+    run as they are; the weighted sum of latents then goes through Wuv_j.  The pages therefore hold what the design
+    says must be kept, c and kr, and nothing a head.  `position` turns the first `position.rotary_dim` of the rot_dim
+    coordinates.  `names`: the tensors' names under `name`."""
+
+    NAMES = {"q": "q", "dq": "dq", "dq_norm": "dq.norm", "uq": "uq", "dkv": "dkv", "dkv_norm": "dkv.norm", "uk": "uk",
+             "uv": "uv", "gate": "g", "o": "o"}
+
+    def __init__(self, name, hidden, heads, dim, rot_dim, vdim, kv_rank, scale, eps, position, q_rank=None, window=None,
+                 head_gate=True, names=None, tuning=None):
+        self.pad = -(-(kv_rank + rot_dim) // 8) * 8
+        if self.pad > 256:
+            raise ValueError(f"a latent of {kv_rank} and {rot_dim} turning coordinates: at most 256 together")
+        if not scale > 0:
+            raise ValueError("the score scale must be positive")
+        if position.rotary_dim > rot_dim:
+            raise ValueError(f"{position.rotary_dim} coordinates turn, the queries and keys have {rot_dim} for it")
+        self.name, self.hidden, self.heads, self.dim, self.rot_dim, self.vdim = name, hidden, heads, dim, rot_dim, vdim
+        self.kv_rank, self.scale, self.eps, self.position = kv_rank, float(scale), float(eps), position
+        self.q_rank, self.window, self.head_gate = q_rank, window, bool(head_gate)
+        self.names = {**self.NAMES, **(names or {})}
+        self.tuning = tuning or kernel.DEFAULT_TUNING
+        self.w_q = self.w_small = self.w_absorb = self.w_value = self.w_out = None
+
+    def _tensor(self, which):
+        return f"{self.name}.{self.names[which]}"
+
+    def kernel_units(self, dtype):
+        return kernel.kernel_units(self.pad, dtype)
+
+    def step_arrays(self):
+        return [kernel.SingleRows(self.tuning.split_single_from), kernel.RowsLongestFirst()]
+
+    def cache_need(self):
+        return KVNeed(1, self.pad, self.window)
+
+    def tensor_specs(self):
+        H, nh, D, R, V, r, t = self.hidden, self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank, self._tensor
+        if self.q_rank is None:
+            specs = [TensorSpec(t("q"), (nh * (D + R), H))]
+        else:
+            specs = [TensorSpec(t("dq"), (self.q_rank, H)), TensorSpec(t("dq_norm"), (self.q_rank,), init="one_plus_normal"),
+                     TensorSpec(t("uq"), (nh * (D + R), self.q_rank))]
+        specs += [TensorSpec(t("dkv"), (r + R, H)), TensorSpec(t("dkv_norm"), (r,), init="one_plus_normal"),
+                  TensorSpec(t("uk"), (nh * D, r)), TensorSpec(t("uv"), (nh * V, r)), TensorSpec(t("o"), (H, nh * V))]
+        if self.head_gate:
+            specs.append(TensorSpec(t("gate"), (nh, H)))
+        return specs
+
+    def bind(self, tensors, dtype):
+        nh, D, V, r, t = self.heads, self.dim, self.vdim, self.kv_rank, self._tensor
+        # one product with float results for everything small that reads the mixer's input: the latents before their
+        # norms, the key part that turns, the gates; the queries' own (large) product gives the compute dtype
+        small = ([] if self.q_rank is None else ["dq"]) + ["dkv"] + (["gate"] if self.head_gate else [])
+        parts = [matrix_operand(tensors[t(p)], dtype) for p in small]
+        rows = sum(p.shape[0] for p in parts)
+        if rows % 8:
+            parts.append(torch.zeros(8 - rows % 8, self.hidden, dtype=parts[0].dtype, device=parts[0].device))
+        self.w_small = torch.cat(parts, dim=0).contiguous()
+        self.w_q = matrix_operand(tensors[t("q" if self.q_rank is None else "uq")], dtype)
+        self.w_absorb = matrix_operand(tensors[t("uk")], dtype).view(nh, D, r).transpose(1, 2).contiguous()   # [heads, rank, dim]
+        self.w_value = matrix_operand(tensors[t("uv")], dtype).view(nh, V, r).contiguous()                    # [heads, vdim, rank]
+        self.w_out = matrix_operand(tensors[t("o")], dtype)
+        self.kv_weight = tensors[t("dkv_norm")].to(torch.float32).contiguous()
+        self.q_weight = None if self.q_rank is None else tensors[t("dq_norm")].to(torch.float32).contiguous()
+        self.q_size = 0
+        if self.q_rank is not None:        # (the query latent's size may be the file's to say: both halves must agree)
+            self.q_size = tensors[t("dq")].shape[0]
+            if self.w_q.shape[1] != self.q_size or self.q_weight.shape[0] != self.q_size:
+                raise ValueError(f"{self.name}: the query latent's projections and norm disagree about its size")
+
+    def prepare(self, device, dtype):
+        self.position.prepare(device, dtype)
+
+    def forward(self, h, residual, ctx, site, norm=None):
+        T = h.shape[0]
+        nh, D, R, V, r, pad = self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank, self.pad
+        gid, kcache, vcache = ctx.cache.pages_of_site(site)
+        view = ctx.kv[gid]
+        cos, sin = self.position.tables()
+        small = ops.gemm(h, self.w_small, ctx.buffer("lat.small", (T, self.w_small.shape[0]), torch.float32), scratch=ctx.scratch)
+        first = 0
+        if self.q_rank is not None:
+            cq = ops.rms_slice(small[:, :self.q_size], self.q_weight, ctx.buffer("lat.cq", (T, self.q_size), ctx.dtype), self.eps)
+            h, first = cq, self.q_size
+        q = ops.gemm(h, self.w_q, ctx.buffer("lat.q", (T, nh * (D + R)), ctx.dtype), scratch=ctx.scratch)
+        qa = ctx.buffer("lat.qa", (T, nh * pad), ctx.dtype)
+        ops.latent_keys(small[:, first:first + r + R], self.kv_weight, q, qa, kcache, vcache, ctx.positions, view.slots, cos, sin,
+                        nh, D, R, r, pad, view.page_size, self.eps, interleaved=self.position.pairing == "interleaved")
+        ops.heads_product(q, D + R, self.w_absorb, qa, pad)
+        out = ctx.buffer("lat.out", (T, nh * pad), ctx.dtype)
+        kernel.paged_attention(ctx, qa, nh * pad, kcache, vcache, view, out, nh, 1, pad, self.window, self.scale, tuning=self.tuning)
+        gates = small[:, first + r + R:first + r + R + nh] if self.head_gate else None
+        act = ops.heads_product(out, pad, self.w_value, ctx.buffer("lat.act", (T, nh * V), ctx.dtype), V, gate=gates)
+        return ctx.add_product(act, self.w_out, residual)
+
+
 register_part("mixer", "attention", PagedAttention)
+register_part("mixer", "latent_attention", LatentAttention)
 register_part("mixer", "normed_gated_attention", NormedGatedAttention)

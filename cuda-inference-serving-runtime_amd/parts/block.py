@@ -7,11 +7,14 @@ from .base import Part, register_part
 
 
 class PreNormBlock(Part):
-    def __init__(self, mixer_norm, mixer, ffn_norm, ffn):
+    def __init__(self, mixer_norm, mixer, ffn_norm=None, ffn=None):
+        """`ffn` None (and no `ffn_norm`): a layer without a feed-forward."""
+        if (ffn is None) != (ffn_norm is None):
+            raise ValueError("a feed-forward comes with the norm before it, or not at all")
         self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
 
     def parts(self):
-        return [self.mixer_norm, self.mixer, self.ffn_norm, self.ffn]
+        return [p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn) if p is not None]
 
     def tensor_specs(self):
         return [s for p in self.parts() for s in p.tensor_specs()]
@@ -51,13 +54,15 @@ class PreNormBlock(Part):
         # ctx.next_norm names the norm that reads the residual stream after the part that runs: a part's last
         # product may be left to it (ctx.add_product); on entry it is the norm after this block
         after = ctx.next_norm
-        ffn_fuses = self.ffn.fuses_norm(self.ffn_norm, residual, ctx)
-        ctx.next_norm = None if ffn_fuses else self.ffn_norm
+        ffn_fuses = self.ffn is not None and self.ffn.fuses_norm(self.ffn_norm, residual, ctx)
+        ctx.next_norm = after if self.ffn is None else None if ffn_fuses else self.ffn_norm
         if self.mixer.fuses_norm(self.mixer_norm, residual, ctx):
             ctx.settle(residual)
             residual = self.mixer.forward(None, residual, ctx, site, norm=self.mixer_norm)
         else:
             residual = self.mixer.forward(self.mixer_norm.forward(residual, ctx), residual, ctx, site)
+        if self.ffn is None:
+            return residual
         if ffn_fuses:
             ctx.settle(residual)
             ctx.next_norm = after

@@ -92,5 +92,39 @@ class ClampedGLU(FeedForward):
         return add_sublayer(residual, self.output(h, ctx), None, 1.0)
 
 
+class DenseMLP(FeedForward):
+    """y = act(h Wu^T) Wd^T, one matrix up and one down, no gate.  `activation`: "gelu" (the exact form, with the error
+    function) or "gelu_tanh".  `names` = (up, down), the tensors' names under `name`."""
+
+    def __init__(self, name, hidden, intermediate, activation="gelu", names=("up", "down")):
+        if activation not in ops.GELU_KINDS:
+            raise ValueError(f"activation {activation!r}: one of {sorted(ops.GELU_KINDS)}")
+        self.name, self.hidden, self.intermediate, self.activation = name, hidden, intermediate, activation
+        self.names = tuple(names)
+        self.w_up = self.w_down = None
+
+    def _tensor(self, which):
+        return f"{self.name}.{self.names[which]}"
+
+    def tensor_specs(self):
+        return [TensorSpec(self._tensor(0), (self.intermediate, self.hidden)), TensorSpec(self._tensor(1), (self.hidden, self.intermediate))]
+
+    def bind(self, tensors, dtype):
+        self.w_up, self.w_down = (matrix_operand(tensors[self._tensor(i)], dtype) for i in (0, 1))
+
+    def _activations(self, h, ctx):
+        T = h.shape[0]
+        up = ops.gemm(h, self.w_up, ctx.buffer("ffn.up", (T, self.intermediate), ctx.dtype), scratch=ctx.scratch)
+        return ops.gelu(up, ctx.buffer("ffn.act", (T, self.intermediate), ctx.dtype), self.activation)
+
+    def output(self, h, ctx):
+        """The feed-forward's result, float [T, hidden], without the residual sum."""
+        return ctx.product_for_norm(self._activations(h, ctx), self.w_down, "ffn.out")
+
+    def forward(self, h, residual, ctx, norm=None):
+        return ctx.add_product(self._activations(h, ctx), self.w_down, residual)
+
+
 register_part("ffn", "gated_mlp", GatedMLP)
+register_part("ffn", "dense_mlp", DenseMLP)
 register_part("ffn", "clamped_glu", ClampedGLU)

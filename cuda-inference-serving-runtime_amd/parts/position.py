@@ -11,6 +11,8 @@ What a position part gives a mixer: `tables() -> (cos, sin)` float
 is, "split_half" (i, i + pairs) or "interleaved" (2i, 2i + 1).  A part without
 the attribute is split-half.
 """
+import math
+
 import numpy as np
 import torch
 
@@ -18,7 +20,12 @@ from .base import Part, register_part
 
 
 class RotaryEmbedding(Part):
-    def __init__(self, head_dim, theta, max_positions, rotary_dim=None, pairing="split_half"):
+    def __init__(self, head_dim, theta, max_positions, rotary_dim=None, pairing="split_half", scaling=None):
+        """`scaling` (YaRN): {"factor", "original", "fast", "slow"}.  With turns(t) the index of the pair that makes t
+        turns over `original` positions, rotary_dim * ln(original / (2 pi t)) / (2 ln theta), pairs up to
+        lo = max(floor(turns(fast)), 0) keep their frequency, pairs from hi = min(ceil(turns(slow)), rotary_dim - 1) on
+        turn `factor` times slower, those between go over linearly; cosines and sines are multiplied by
+        0.1 ln(factor) + 1."""
         if pairing not in ("split_half", "interleaved"):
             raise ValueError(f"pairing {pairing!r} is neither split_half nor interleaved")
         self.pairing = pairing
@@ -26,19 +33,45 @@ class RotaryEmbedding(Part):
         self.rotary_dim = head_dim if rotary_dim is None else rotary_dim
         if self.rotary_dim % 2 or not 0 < self.rotary_dim <= head_dim:
             raise ValueError(f"rotary size {self.rotary_dim} must be even and at most the head size {head_dim}")
+        self.scaling = None
+        if scaling is not None:
+            missing = [k for k in ("factor", "original", "fast", "slow") if k not in scaling]
+            if missing:
+                raise ValueError(f"rotary scaling lacks {missing}")
+            self.scaling = {k: float(scaling[k]) for k in ("factor", "original", "fast", "slow")}
+            if not (self.scaling["factor"] > 0 and self.scaling["original"] > 0 and self.scaling["fast"] > 0 and self.scaling["slow"] > 0):
+                raise ValueError("rotary scaling: factor, original, fast and slow must be positive")
         self._tables = None
 
+    def frequencies(self):
+        """Radians a position of each pair (float64 [rotary_dim / 2])."""
+        half, dims = self.rotary_dim // 2, self.rotary_dim
+        index = np.arange(half, dtype=np.float64)
+        freq = np.float64(self.theta) ** (-index * 2.0 / dims)
+        s = self.scaling
+        if s is None:
+            return freq
+
+        def turns(t):
+            return dims * math.log(s["original"] / (2.0 * math.pi * t)) / (2.0 * math.log(self.theta))
+
+        lo, hi = max(math.floor(turns(s["fast"])), 0), min(math.ceil(turns(s["slow"])), dims - 1)
+        ramp = np.clip((index - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        return freq / s["factor"] * ramp + freq * (1.0 - ramp)
+
+    def magnitude(self):
+        """What cosines and sines are multiplied by (1 without scaling)."""
+        return 1.0 if self.scaling is None else 0.1 * math.log(self.scaling["factor"]) + 1.0
+
     def angles(self):
-        half = self.rotary_dim // 2
-        inv_freq = np.float64(self.theta) ** (-np.arange(half, dtype=np.float64) * 2.0 / self.rotary_dim)
-        return np.arange(self.max_positions, dtype=np.float64)[:, None] * inv_freq[None, :]
+        return np.arange(self.max_positions, dtype=np.float64)[:, None] * self.frequencies()[None, :]
 
     def prepare(self, device, dtype):
         if self._tables is not None and self._tables[0].device == torch.device(device):
             return                      # one part may serve many layers: its tables are built once
-        a = self.angles()
-        self._tables = (torch.from_numpy(np.cos(a).astype(np.float32)).to(device).contiguous(),
-                        torch.from_numpy(np.sin(a).astype(np.float32)).to(device).contiguous())
+        a, m = self.angles(), self.magnitude()
+        self._tables = (torch.from_numpy((np.cos(a) * m).astype(np.float32)).to(device).contiguous(),
+                        torch.from_numpy((np.sin(a) * m).astype(np.float32)).to(device).contiguous())
 
     def tables(self):
         return self._tables

@@ -12,6 +12,12 @@ the state in the cache manager's state slots, in float in every mode:
                          causal convolution with silu whose last inputs are part of the state; y = o + D x, times
                          silu(z), RMS-normed in equal parts of the row, then the output projection.
 
+  GatedDeltaRule         S <- g_t S; u = beta_t (v_t - S^T k_t); S <- S + k_t u^T; o_t = S^T q_t, a kernel of its own
+                         (ops.delta_scan): g_t = exp(-exp(A_log) softplus(a_t + dt_bias)) and beta_t = sigmoid(b_t) one
+                         number a head; q, k, v come out of a short causal convolution with silu (its last inputs are
+                         part of the state), q and k are made unit vectors per head, q scaled by dim^(-1/2); each
+                         head's result RMS-normed, times silu of a gate projection, then the output projection.
+
 The projections and the convolution's inputs are products with float results; decays, step sizes, gates of the
 recurrence and the norms are float arithmetic; the operands of the output projections are the compute dtype.
 """
@@ -162,6 +168,89 @@ class StateSpaceDuality(Mixer):
         return add_sublayer(residual, self.output(h, ctx, site), None, 1.0)
 
 
+class GatedDeltaRule(Mixer):
+    """The gated delta rule.  `kv_heads` heads of q and k (`dim` each) serve `heads` heads of v (`vdim` each), head j
+    using q/k head j // (heads / kv_heads).  `names`: the tensors' names under `name`; the convolutions' taps are
+    `<projection>.conv`, [channels, taps], the last column the current token's."""
+
+    NAMES = {"q": "q", "k": "k", "v": "v", "write": "b", "decay": "a", "dt_bias": "dt_bias", "a_log": "A_log", "gate": "g",
+             "norm": "norm", "o": "o", "conv": "conv"}
+    MAX_TAPS = 16
+
+    def __init__(self, name, hidden, heads, kv_heads, dim, vdim, taps, eps, unit_eps=1e-6, names=None):
+        if heads % kv_heads:
+            raise ValueError(f"{heads} heads are not a multiple of {kv_heads} query/key heads")
+        if not 1 <= taps <= self.MAX_TAPS:
+            raise ValueError(f"a convolution of {taps} taps: 1 to {self.MAX_TAPS}")
+        if dim > 256:
+            raise ValueError(f"query/key heads of {dim}: at most 256")
+        self.name, self.hidden, self.heads, self.kv_heads, self.dim, self.vdim = name, hidden, heads, kv_heads, dim, vdim
+        self.taps, self.eps, self.unit_eps = int(taps), float(eps), float(unit_eps)
+        self.qk, self.inner = kv_heads * dim, heads * vdim
+        self.channels = 2 * self.qk + self.inner           # what the convolution runs over: q, k, v
+        self.names = {**self.NAMES, **(names or {})}
+
+    def _tensor(self, which):
+        return f"{self.name}.{self.names[which]}"
+
+    def kernel_units(self, dtype):
+        return [library.RECURRENCE]
+
+    def state_need(self):
+        """One float row a request: the heads' states [heads, dim, vdim], then the convolution's last taps - 1 inputs
+        [taps - 1, channels]."""
+        return StateNeed((self.heads * self.dim * self.vdim + (self.taps - 1) * self.channels,), "float32")
+
+    def tensor_specs(self):
+        H, t, conv = self.hidden, self._tensor, self.names["conv"]
+        return [TensorSpec(t("q"), (self.qk, H)), TensorSpec(t("k"), (self.qk, H)), TensorSpec(t("v"), (self.inner, H)),
+                TensorSpec(f"{t('q')}.{conv}", (self.qk, self.taps)), TensorSpec(f"{t('k')}.{conv}", (self.qk, self.taps)),
+                TensorSpec(f"{t('v')}.{conv}", (self.inner, self.taps)),
+                TensorSpec(t("write"), (self.heads, H)), TensorSpec(t("decay"), (self.heads, H)),
+                TensorSpec(t("dt_bias"), (self.heads,)), TensorSpec(t("a_log"), (self.heads,)),
+                TensorSpec(t("gate"), (self.inner, H)), TensorSpec(t("norm"), (self.vdim,), init="one_plus_normal"),
+                TensorSpec(t("o"), (H, self.inner))]
+
+    def bind(self, tensors, dtype):
+        t, conv = self._tensor, self.names["conv"]
+        # one product with float results: [q | k | v | decay | write | gate] (everything that enters the recurrence is float)
+        parts = [matrix_operand(tensors[t(p)], dtype) for p in ("q", "k", "v", "decay", "write", "gate")]
+        rows = sum(p.shape[0] for p in parts)
+        if rows % 8:
+            parts.append(torch.zeros(8 - rows % 8, self.hidden, dtype=parts[0].dtype, device=parts[0].device))
+        self.w_in = torch.cat(parts, dim=0).contiguous()
+        self.w_out = matrix_operand(tensors[t("o")], dtype)
+        self.conv = torch.cat([_float(tensors[f"{t(p)}.{conv}"]) for p in ("q", "k", "v")], dim=0).contiguous()
+        self.dt_bias, self.a_log = _float(tensors[t("dt_bias")]), _float(tensors[t("a_log")])
+        self.norm_weight = _float(tensors[t("norm")])
+
+    def _normed_result(self, h, ctx, site):
+        """The operand of the output projection [T, heads * vdim]; moves the request's state on."""
+        T = h.shape[0]
+        qk, inner, ch, nh = self.qk, self.inner, self.channels, self.heads
+        proj = ops.gemm(h, self.w_in, ctx.buffer("delta.proj", (T, self.w_in.shape[0]), torch.float32), scratch=ctx.scratch)
+        state = ctx.cache.state_storage[site]
+        heads_state = nh * self.dim * self.vdim
+        qkv = ctx.buffer("delta.qkv", (T, ch), torch.float32)
+        step, decay = ctx.buffer("delta.step", (T, nh), torch.float32), ctx.buffer("delta.decay", (T, nh), torch.float32)
+        ops.conv_silu(proj[:, :ch], self.conv, None, state[:, heads_state:], qkv, ctx.seg_of_row, ctx.seg_start, ctx.state_slots,
+                      gates=(proj[:, ch:ch + nh], self.dt_bias, self.a_log, step, decay))
+        ops.unit_heads(qkv[:, :2 * qk], 2 * self.kv_heads, self.dim, eps=self.unit_eps)
+        o = ctx.buffer("delta.o", (T, inner), torch.float32)
+        ops.delta_scan(qkv[:, :qk], qkv[:, qk:2 * qk], qkv[:, 2 * qk:], decay, proj[:, ch + nh:ch + 2 * nh], o, state,
+                       ctx.seg_start, ctx.state_slots, nh, self.dim, self.vdim, share=nh // self.kv_heads, q_scale=self.dim ** -0.5)
+        act = ops.group_norm_gate(o, proj[:, ch + 2 * nh:ch + 2 * nh + inner], self.norm_weight, ctx.buffer("delta.act", (T, inner), ctx.dtype),
+                                  nh, self.eps, gate_first=False, shared_weight=True)
+        return act
+
+    def output(self, h, ctx, site):
+        """The mixer's result, float [T, hidden], without the residual sum."""
+        return ctx.product_for_norm(self._normed_result(h, ctx, site), self.w_out, "delta.y")
+
+    def forward(self, h, residual, ctx, site, norm=None):
+        return ctx.add_product(self._normed_result(h, ctx, site), self.w_out, residual)
+
+
 class SideBySide(Mixer):
     """Two mixers that read the same input; the result is half the sum of theirs, each RMS-normed over the model
     width with a weight of its own (`<name>.<first_out>` / `<name>.<second_out>`).  At most one of the two keeps pages
@@ -215,3 +304,4 @@ class SideBySide(Mixer):
 register_part("mixer", "gated_linear_attention", GatedLinearAttention)
 register_part("mixer", "state_space_duality", StateSpaceDuality)
 register_part("mixer", "side_by_side", SideBySide)
+register_part("mixer", "gated_delta_rule", GatedDeltaRule)
