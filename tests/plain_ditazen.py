@@ -218,3 +218,12 @@ def read_folder(folder):
     config = json.loads((folder / "config.json").read_text())
     tensors = {k: v.to(torch.float64).numpy() for k, v in load_file(str(folder / "model.safetensors")).items()}
     return config, tensors
+
+
+def greedy(config, w, prompt, n_new):
+    """The tokens that picking the largest logit generates after `prompt` (the lowest index wins a tie)."""
+    tokens, new = list(prompt), []
+    for _ in range(n_new):
+        new.append(int(np.argmax(forward(config, w, tokens)[-1])))
+        tokens.append(new[-1])
+    return new
