@@ -283,6 +283,7 @@ def main():
     ap.add_argument("--check", type=int, default=1, choices=[0, 1], help="compare the timed way of running with the plain one first")
     ap.add_argument("--widths", default="1024,2048,4096", help="designs workload: model widths to time (comma separated)")
     ap.add_argument("--design-layers", type=int, default=4, help="designs workload: layers of each model")
+    ap.add_argument("--designs", default="llama,novosun,ditazen", help="designs workload: which designs to time (comma separated)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only; --gpus {args.gpus} is not run")
@@ -387,7 +388,7 @@ def main():
 
 
 def design_configs(width, layers, context):
-    """A Llama and a Novosun configuration of the same width, depth, feed-forward size and vocabulary.  The Novosun
+    """A Llama, a Novosun and a Ditazen configuration of the same width, depth, feed-forward size and vocabulary.  The Novosun
     layers alternate: softmax attention (heads of 64 for keys, 128 for values, a quarter as many key/value heads) beside
     a state-space layer (inner size twice the width in heads of 64, 128 states, a convolution of 4 taps), then gated
     linear attention (key size half the width, value size the width, in heads of 128 x 256)."""
@@ -403,11 +404,23 @@ def design_configs(width, layers, context):
     gla = {"type": "gla", "mlp": mlp, "mixer": {"heads": width // 256, "dim": 128, "vdim": 256, "tau": 16.0}}
     novosun = {"architecture": "Novosun", "vocab": vocab, "width": width, "residual_mult": 0.5, "norm": {"eps": 1e-5},
                "layers": [side if i % 2 == 0 else gla for i in range(layers)], "max_positions": context}
-    return {"llama": llama, "novosun": novosun}
+    # Ditazen: latent attention through a query latent over every earlier key, the gated delta rule (twice as many value
+    # heads as query/key heads, all of 128, a convolution of 4 taps), latent attention over a window of 1,024 keys, the
+    # delta rule again; latents of 192 with 64 turning coordinates, heads of 128; feed-forwards of one matrix up and one down
+    dense = {"kind": "dense", "ff": ff}
+    heads = width // 128
+    lat = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 192, "scale": 192 ** -0.5}
+    first = {"type": "latent_attention_2", "mlp": dense, "mixer": {**lat, "q_rank": 3 * width // 4, "rot": {
+        "base": 10000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}}
+    window = {"type": "latent_attention", "mlp": dense, "mixer": {**lat, "rot": {"base": 10000.0, "dims": 64}, "mask": {"size": 1024}}}
+    rule = {"type": "delta", "mlp": dense, "mixer": {"heads": 2 * heads, "kv_heads": heads, "dim": 128, "vdim": 128, "conv": 4}}
+    ditazen = {"architecture": "Ditazen", "vocab": vocab, "width": width, "logit_scale": 1.0, "norm": {"eps": 1e-5},
+               "layers": [(first, rule, window, rule)[i % 4] for i in range(layers)], "max_positions": context}
+    return {"llama": llama, "novosun": novosun, "ditazen": ditazen}
 
 
 def designs(args):
-    """Prompt steps and decode steps of the Novosun design beside the Llama design at equal width, depth, feed-forward
+    """Prompt steps and decode steps of the Novosun and Ditazen designs beside the Llama design at equal width, depth, feed-forward
     size and vocabulary (random weights drawn on the device): tokens a second of a whole prompt of --prompt tokens and
     of decode steps of 1, 8 and 64 requests after such prompts, through the step function with captured programs and
     the greedy pick."""
@@ -424,6 +437,8 @@ def designs(args):
     out = {}
     for width in [int(w) for w in args.widths.split(",") if w]:
         for design, raw in design_configs(width, args.design_layers, context).items():
+            if design not in args.designs.split(","):
+                continue
             torch.cuda.empty_cache()
             model = random_model(raw, seed=0, dtype=args.dtype)
             parameters = sum(int(np.prod(s.drawn_shape())) for s in model.tensor_specs())
@@ -460,7 +475,7 @@ def designs(args):
             result["prefill"] = {"tokens": prompt, "ms": round(pf * 1e3, 3), "tokens_per_s": round(prompt / pf, 1)}
             out.setdefault(str(width), {})[design] = result
             del runner, model
-    return {"metric": f"prompt and decode tokens/s of the Novosun design beside Llama at equal width, {args.design_layers} layers",
+    return {"metric": f"prompt and decode tokens/s of the Novosun and Ditazen designs beside Llama at equal width, {args.design_layers} layers",
             "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "steps": steps,
             "data": "synthetic (random weights N(0,0.02), uniform-random token ids)", "prompt_len": prompt,
             "execution": args.execution, "widths": out}

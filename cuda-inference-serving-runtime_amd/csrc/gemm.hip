@@ -127,11 +127,20 @@ __host__ __device__ inline int patch_side(int tiles) {
 // column tiles take gate rows and its last TN/2 the up rows of the same output columns, so a lane ends
 // with gate and up of one output element in its registers and writes silu(gate) * up (both rounded to
 // bf16 first, as the two-kernel path does); a block then covers BN/2 output columns.
+// A batch of products in one launch (grid.y of them): product h reads A + h a, W + h w and writes C + h c (elements);
+// with `gate`, row m of product h is multiplied by sigmoid(gate[m * ldg + h]).  Zeros: one product, no gate.
+struct HeadBatch { long long a, w, c; const float* gate; int ldg; };
+
 template <int TM, int TN, int BK, typename TC, bool VEC, bool SWIGLU = false, int WM = 2>
 __global__ void __launch_bounds__(WM * 128)
 gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
-                 TC* C, int ldc, const float* R, int ldr, int M, int N, int K, int dual_off = 0, GateLaw law = {}) {
+                 TC* C, int ldc, const float* R, int ldr, int M, int N, int K, int dual_off = 0, GateLaw law = {},
+                 HeadBatch heads = {}) {
     static_assert(!SWIGLU || (TN % 2 == 0 && VEC), "the activation pairs column tiles");
+    // blockIdx.y: which of a batch of products with a matrix of its own each (one launch for all heads)
+    A += (size_t)blockIdx.y * heads.a;
+    W += (size_t)blockIdx.y * heads.w;
+    C += (size_t)blockIdx.y * heads.c;
     constexpr int BM = WM * TM * 16, BN = 2 * TN * 16, NT = WM * 128;   // WM x 2 waves
     constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;           // output columns a block covers
     constexpr int CPR = BK / 8;                            // 16-byte chunks per tile row
@@ -274,6 +283,17 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
                 for (int e = 0; e < 4; ++e) acc[i][j][e] += rv[e];
             }
     }
+    if (heads.gate) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int m = min(m0 + wm * TM * 16 + i * 16 + g * 4 + e, M - 1);
+                const float s = 1.0f / (1.0f + expf(-heads.gate[(size_t)m * heads.ldg + blockIdx.y]));
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j][e] *= s;
+            }
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -297,18 +317,20 @@ static long long tile_slots(long long tiles_m, long long tiles_n) {
 
 template <int TM, int TN, int BK, int WM = 2>
 static int launch_bf16(const bf16_t* A, int lda, const bf16_t* W, int ldw, void* C, int ldc, const float* R,
-                       int ldr, int M, int N, int K, int out_dtype, hipStream_t stream) {
+                       int ldr, int M, int N, int K, int out_dtype, hipStream_t stream, HeadBatch heads = {}, int n_heads = 1) {
     constexpr int BM = WM * TM * 16, BN = 2 * TN * 16, NT = WM * 128;
     const long long slots = tile_slots((M + BM - 1) / BM, (N + BN - 1) / BN);
-    if (slots > (1ll << 30)) return (int)hipErrorInvalidValue;
-    dim3 grid((unsigned)((slots + 7) / 8 * 8));
-    const bool vec = lda % 8 == 0 && ldw % 8 == 0 && K % 8 == 0 && ((uintptr_t)A) % 16 == 0 && ((uintptr_t)W) % 16 == 0;
+    if (slots > (1ll << 30) || n_heads < 1 || n_heads > 65535) return (int)hipErrorInvalidValue;
+    dim3 grid((unsigned)((slots + 7) / 8 * 8), n_heads);
+    const bool vec = lda % 8 == 0 && ldw % 8 == 0 && K % 8 == 0 && ((uintptr_t)A) % 16 == 0 && ((uintptr_t)W) % 16 == 0 &&
+                     heads.a % 8 == 0 && heads.w % 8 == 0;
+    const GateLaw law{};
     if (out_dtype == DT_F32) {
-        if (vec) gemm_bf16_kernel<TM, TN, BK, float, true, false, WM><<<grid, NT, 0, stream>>>(A, lda, W, ldw, (float*)C, ldc, R, ldr, M, N, K);
-        else gemm_bf16_kernel<TM, TN, BK, float, false, false, WM><<<grid, NT, 0, stream>>>(A, lda, W, ldw, (float*)C, ldc, R, ldr, M, N, K);
+        if (vec) gemm_bf16_kernel<TM, TN, BK, float, true, false, WM><<<grid, NT, 0, stream>>>(A, lda, W, ldw, (float*)C, ldc, R, ldr, M, N, K, 0, law, heads);
+        else gemm_bf16_kernel<TM, TN, BK, float, false, false, WM><<<grid, NT, 0, stream>>>(A, lda, W, ldw, (float*)C, ldc, R, ldr, M, N, K, 0, law, heads);
     } else {
-        if (vec) gemm_bf16_kernel<TM, TN, BK, bf16_t, true, false, WM><<<grid, NT, 0, stream>>>(A, lda, W, ldw, (bf16_t*)C, ldc, R, ldr, M, N, K);
-        else gemm_bf16_kernel<TM, TN, BK, bf16_t, false, false, WM><<<grid, NT, 0, stream>>>(A, lda, W, ldw, (bf16_t*)C, ldc, R, ldr, M, N, K);
+        if (vec) gemm_bf16_kernel<TM, TN, BK, bf16_t, true, false, WM><<<grid, NT, 0, stream>>>(A, lda, W, ldw, (bf16_t*)C, ldc, R, ldr, M, N, K, 0, law, heads);
+        else gemm_bf16_kernel<TM, TN, BK, bf16_t, false, false, WM><<<grid, NT, 0, stream>>>(A, lda, W, ldw, (bf16_t*)C, ldc, R, ldr, M, N, K, 0, law, heads);
     }
     return CISR_LAUNCH_CHECK();
 }
@@ -392,6 +414,30 @@ extern "C" int cisr_gemm_bf16_tile(const void* A, int lda, const void* W, int ld
         GEMM_TILE(1, 1, 2) GEMM_TILE(1, 2, 2) GEMM_TILE(2, 2, 2) GEMM_TILE(4, 2, 2) GEMM_TILE(4, 4, 2)
     }
 #undef GEMM_TILE
+    return (int)hipErrorInvalidValue;
+}
+
+// A product a head in one launch: C[m, h * c_head + n] = sum_k A[m, h * a_head + k] W[h][n][k] (W [heads, N, K] contiguous),
+// times sigmoid(gate[m * ldg + h]) where `gate` is given.  bf16 operands, bf16 or float results.
+extern "C" int cisr_gemm_bf16_heads(const void* A, int lda, int a_head, const void* W, void* C, int ldc, int c_head,
+                                    const float* gate, int ldg, int M, int N, int K, int heads, int out_dtype, hipStream_t stream) {
+    if (M <= 0 || N <= 0 || heads <= 0) return 0;
+    if (K <= 0) return (int)hipErrorInvalidValue;
+    const bf16_t* a = (const bf16_t*)A; const bf16_t* w = (const bf16_t*)W;
+    const HeadBatch batch{a_head, (long long)N * K, c_head, gate, ldg};
+    auto blocks = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn) * heads; };
+    int tile;
+    if (M <= 32) tile = 122;
+    else if (blocks(128, 128) >= 512) tile = 442;
+    else if (blocks(128, 64) >= 512) tile = 422;
+    else if (blocks(64, 64) < 256) tile = 122;
+    else tile = 222;
+#define HEADS_TILE(TM, TN, WM) \
+    case TM * 100 + TN * 10 + WM: return launch_bf16<TM, TN, 64, WM>(a, lda, w, K, C, ldc, nullptr, 0, M, N, K, out_dtype, stream, batch, heads);
+    switch (tile) {
+        HEADS_TILE(1, 2, 2) HEADS_TILE(2, 2, 2) HEADS_TILE(4, 2, 2) HEADS_TILE(4, 4, 2)
+    }
+#undef HEADS_TILE
     return (int)hipErrorInvalidValue;
 }
 

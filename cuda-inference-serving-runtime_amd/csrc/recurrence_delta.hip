@@ -7,7 +7,8 @@
 // columns of S go their own ways (column c needs k, q, v_t[c] and itself only), so a head is as many waves as it has
 // tiles of columns.  Both products with the state are taken from the state as the row finds it,
 //   S^T k = g (S_old^T k),   o = g (S_old^T q) + (k . q) u,
-// so that a row costs one meeting of the lanes that share a column instead of two.
+// so that a row costs one meeting of the lanes that share a column instead of two.  The lanes that share a column are
+// neighbours, so their sums meet by moves inside a row of 16 lanes, without a trip through LDS.
 // With it: the unit vectors x / sqrt(sum(x^2) + eps) * scale of the heads of a row (q and k of this rule).
 #include "common.h"
 
@@ -26,17 +27,36 @@ struct DeltaArgs {
 
 #define DELTA_GROUP_OF(RPT) ((RPT) >= 32 ? 4 : 8)
 
-// A wave a (segment, head, tile of COLS columns); a lane owns two neighbouring columns and the rows
-// l / (COLS / 2) + NG i, i < RPT, NG = 128 / COLS, of the state in registers.  Rows of a segment are walked in order,
-// GROUP at a time through LDS, the next group's loads in flight while this one is walked.
-template <int COLS, int RPT>
+// The sum of x over the NG (4, 8 or 16) neighbouring lanes of an aligned group, in every lane of the group, by
+// data-parallel-primitive moves inside a row of 16 lanes: neighbours, pairs, then the mirror image of a half row and
+// of a row (the partial sums are by then the same in all lanes of a quad, of a half row).
+template <int CTRL>
+__device__ __forceinline__ float lanes_moved(float x) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, false));
+}
+
+template <int NG>
+__device__ __forceinline__ float group_sum(float x) {
+    x += lanes_moved<0xB1>(x);                   // quad_perm [1, 0, 3, 2]
+    x += lanes_moved<0x4E>(x);                   // quad_perm [2, 3, 0, 1]
+    if (NG >= 8) x += lanes_moved<0x141>(x);     // row_half_mirror
+    if (NG >= 16) x += lanes_moved<0x140>(x);    // row_mirror
+    return x;
+}
+
+// A wave a (segment, head, tile of COLS = 128 / NG columns); NG neighbouring lanes share two neighbouring columns, and
+// lane l of them owns the rows l + NG i, i < RPT, of the state in registers.  Rows of a segment are walked in order,
+// GROUP at a time through LDS, the next group's loads in flight while this one is walked; inside a group the next
+// row's operands are read from LDS while this row's sums meet.
+template <int NG, int RPT>
 __global__ void __launch_bounds__(64) delta_scan_kernel(DeltaArgs p) {
-    constexpr int LPG = COLS / 2, NG = WAVE / LPG, GROUP = DELTA_GROUP_OF(RPT), RP = NG * RPT;
-    __shared__ float sq[GROUP * RP], sk[GROUP * RP], sg[GROUP], sb[GROUP], sv[GROUP * 2 * WAVE];
+    constexpr int LPG = WAVE / NG, COLS = 2 * LPG, GROUP = DELTA_GROUP_OF(RPT), RP = NG * RPT;
+    __shared__ float sq[GROUP * RP], sk[GROUP * RP], sg[GROUP], sb[GROUP], sv[GROUP * COLS];
     const int seg = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
     const int t0 = p.seg_start[seg], t1 = p.seg_start[seg + 1];
     if (t1 <= t0) return;
-    const int c = blockIdx.z * COLS + 2 * (lane % LPG), rg = lane / LPG;
+    const int pair = lane / NG, rg = lane % NG;
+    const int c = blockIdx.z * COLS + 2 * pair;
     const bool ok0 = c < p.C, ok1 = c + 1 < p.C;
     const int c0 = ok0 ? c : p.C - 1, c1 = ok1 ? c + 1 : p.C - 1;
     const int R = p.R, C = p.C;
@@ -51,9 +71,9 @@ __global__ void __launch_bounds__(64) delta_scan_kernel(DeltaArgs p) {
     const float* qh = p.q + (size_t)(head / p.share) * R;
     const float* kh = p.k + (size_t)(head / p.share) * R;
     const float* vh = p.v + (size_t)head * C;
-    constexpr int PF = GROUP * RP / WAVE;
+    constexpr int PF = GROUP * RP / WAVE, PV = (GROUP * COLS + WAVE - 1) / WAVE;
     static_assert(GROUP * RP % WAVE == 0, "a group's rows divide among the lanes");
-    float fq[PF], fk[PF], fv[2 * GROUP], fg[GROUP], fb[GROUP];
+    float fq[PF], fk[PF], fv[PV], fg = 0.f, fb = 0.f;
     auto fetch = [&](int tb) {
         const int last = t1 - 1;
 #pragma unroll
@@ -66,12 +86,14 @@ __global__ void __launch_bounds__(64) delta_scan_kernel(DeltaArgs p) {
             fq[j] = in ? qh[t * p.ldq + rr] : 0.f;
         }
 #pragma unroll
-        for (int tt = 0; tt < GROUP; ++tt) {
-            const size_t t = (size_t)min(tb + tt, last);
-            fv[2 * tt] = vh[t * p.ldv + c0];
-            fv[2 * tt + 1] = vh[t * p.ldv + c1];
-            fg[tt] = p.g[t * p.ldg + head];
-            fb[tt] = p.b[t * p.ldb + head];
+        for (int j = 0; j < PV; ++j) {
+            const int idx = lane + WAVE * j, tt = min(idx / COLS, GROUP - 1), cc = blockIdx.z * COLS + idx % COLS;
+            fv[j] = vh[(size_t)min(tb + tt, last) * p.ldv + min(cc, C - 1)];
+        }
+        if (lane < GROUP) {
+            const size_t t = (size_t)min(tb + lane, last);
+            fg = p.g[t * p.ldg + head];
+            fb = p.b[t * p.ldb + head];
         }
     };
     fetch(t0);
@@ -84,51 +106,58 @@ __global__ void __launch_bounds__(64) delta_scan_kernel(DeltaArgs p) {
             sq[lane + WAVE * j] = fq[j];
         }
 #pragma unroll
-        for (int tt = 0; tt < GROUP; ++tt) {
-            sv[(tt * WAVE + lane) * 2] = fv[2 * tt];
-            sv[(tt * WAVE + lane) * 2 + 1] = fv[2 * tt + 1];
-            if (lane == 0) {
-                sg[tt] = fg[tt];
-                sb[tt] = 1.0f / (1.0f + expf(-fb[tt]));
-            }
+        for (int j = 0; j < PV; ++j)
+            if (lane + WAVE * j < GROUP * COLS) sv[lane + WAVE * j] = fv[j];
+        if (lane < GROUP) {
+            sg[lane] = fg;
+            sb[lane] = 1.0f / (1.0f + expf(-fb));
         }
         __syncthreads();
         if (tb + GROUP < t1) fetch(tb + GROUP);
+        float kc[RPT], qc[RPT], v0, v1, g, beta;
+        auto take = [&](int tt) {
+#pragma unroll
+            for (int i = 0; i < RPT; ++i) {
+                kc[i] = sk[tt * RP + rg + NG * i];
+                qc[i] = sq[tt * RP + rg + NG * i];
+            }
+            v0 = sv[tt * COLS + 2 * pair];
+            v1 = sv[tt * COLS + 2 * pair + 1];
+            g = sg[tt];
+            beta = sb[tt];
+        };
+        take(0);
 #pragma unroll 1
         for (int tt = 0; tt < n; ++tt) {
-            const float* qt = sq + tt * RP + rg;
-            const float* kt = sk + tt * RP + rg;
-            const float v0 = sv[(tt * WAVE + lane) * 2], v1 = sv[(tt * WAVE + lane) * 2 + 1];
-            const float g = sg[tt], beta = sb[tt];
             float sk0 = 0.f, sk1 = 0.f, sq0 = 0.f, sq1 = 0.f, kq = 0.f;
 #pragma unroll
             for (int i = 0; i < RPT; ++i) {
-                const float kk = kt[NG * i], qq = qt[NG * i];
-                sk0 += S0[i] * kk;
-                sk1 += S1[i] * kk;
-                sq0 += S0[i] * qq;
-                sq1 += S1[i] * qq;
-                kq += kk * qq;
+                sk0 += S0[i] * kc[i];
+                sk1 += S1[i] * kc[i];
+                sq0 += S0[i] * qc[i];
+                sq1 += S1[i] * qc[i];
+                kq += kc[i] * qc[i];
             }
+            float kn[RPT];
 #pragma unroll
-            for (int off = LPG; off < WAVE; off <<= 1) {
-                sk0 += __shfl_xor(sk0, off, WAVE);
-                sk1 += __shfl_xor(sk1, off, WAVE);
-                sq0 += __shfl_xor(sq0, off, WAVE);
-                sq1 += __shfl_xor(sq1, off, WAVE);
-                kq += __shfl_xor(kq, off, WAVE);
-            }
-            const float u0 = beta * (v0 - g * sk0), u1 = beta * (v1 - g * sk1);
+            for (int i = 0; i < RPT; ++i) kn[i] = kc[i];
+            const float gn = g, bn = beta, w0 = v0, w1 = v1;
+            if (tt + 1 < n) take(tt + 1);                  // the next row's operands are on their way while the sums meet
+            sk0 = group_sum<NG>(sk0);
+            sk1 = group_sum<NG>(sk1);
+            sq0 = group_sum<NG>(sq0);
+            sq1 = group_sum<NG>(sq1);
+            kq = group_sum<NG>(kq);
+            const float u0 = bn * (w0 - gn * sk0), u1 = bn * (w1 - gn * sk1);
 #pragma unroll
             for (int i = 0; i < RPT; ++i) {
-                const float kk = kt[NG * i];
-                S0[i] = g * S0[i] + kk * u0;
-                S1[i] = g * S1[i] + kk * u1;
+                S0[i] = gn * S0[i] + kn[i] * u0;
+                S1[i] = gn * S1[i] + kn[i] * u1;
             }
             if (rg == 0) {
                 float* o = p.out + (size_t)(tb + tt) * p.ldo + (size_t)head * C;
-                if (ok0) o[c] = (g * sq0 + kq * u0) * p.q_scale;
-                if (ok1) o[c + 1] = (g * sq1 + kq * u1) * p.q_scale;
+                if (ok0) o[c] = (gn * sq0 + kq * u0) * p.q_scale;
+                if (ok1) o[c + 1] = (gn * sq1 + kq * u1) * p.q_scale;
             }
         }
     }
@@ -140,34 +169,38 @@ __global__ void __launch_bounds__(64) delta_scan_kernel(DeltaArgs p) {
     }
 }
 
-template <int COLS>
-static int launch_delta_cols(const DeltaArgs& p, int segments, hipStream_t stream) {
-    constexpr int NG = 2 * WAVE / COLS;                           // lanes that share a column
+template <int NG>
+static int launch_delta_group(const DeltaArgs& p, int segments, hipStream_t stream) {
+    constexpr int COLS = 2 * WAVE / NG;
     const int per = (p.R + NG - 1) / NG;                          // rows a lane
     const dim3 grid(segments, p.heads, (p.C + COLS - 1) / COLS);
-    if (per <= 2) delta_scan_kernel<COLS, 2><<<grid, 64, 0, stream>>>(p);
-    else if (per <= 4) delta_scan_kernel<COLS, 4><<<grid, 64, 0, stream>>>(p);
-    else if (per <= 8) delta_scan_kernel<COLS, 8><<<grid, 64, 0, stream>>>(p);
-    else if (per <= 16) delta_scan_kernel<COLS, 16><<<grid, 64, 0, stream>>>(p);
-    else if (per <= 32) delta_scan_kernel<COLS, 32><<<grid, 64, 0, stream>>>(p);
-    else return (int)hipErrorInvalidValue;
+    if (per <= 2) delta_scan_kernel<NG, 2><<<grid, 64, 0, stream>>>(p);
+    else if (per <= 4) delta_scan_kernel<NG, 4><<<grid, 64, 0, stream>>>(p);
+    else if (per <= 8) delta_scan_kernel<NG, 8><<<grid, 64, 0, stream>>>(p);
+    else if (per <= 16) delta_scan_kernel<NG, 16><<<grid, 64, 0, stream>>>(p);
+    else if (per <= 32) {
+        // (32 rows of two columns a lane are what the registers hold; 16 lanes a column reach 256 rows with 16 each)
+        if constexpr (NG <= 8) delta_scan_kernel<NG, 32><<<grid, 64, 0, stream>>>(p);
+        else return (int)hipErrorInvalidValue;
+    } else return (int)hipErrorInvalidValue;
     return CISR_LAUNCH_CHECK();
 }
 
-// cols: 4, 8 or 16 columns a wave (fewer columns are more waves for the same head).
+// cols: 8, 16 or 32 columns a wave (fewer columns are more waves for the same head, and shorter runs of the state);
+// a lane holds at most 32 rows of its columns, so states of more than 128 rows need 16 columns or fewer.
 extern "C" int cisr_delta_scan(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv,
                                const float* g, int ldg, const float* b, int ldb, float* out, int ldo,
                                float* state, long long slot_stride, const int* seg_start, const int* state_slots,
                                int segments, int heads, int R, int C, int share, float q_scale, int cols,
                                hipStream_t stream) {
     if (segments <= 0 || heads <= 0) return 0;
-    if (R <= 0 || C <= 0 || share <= 0 || heads % share || heads > 65535 || segments > 65535 * 32 ||
-        (cols != 4 && cols != 8 && cols != 16) || (C + cols - 1) / cols > 65535 || R > 256)
+    if (R <= 0 || C <= 0 || share <= 0 || heads % share || heads > 65535 || (cols != 8 && cols != 16 && cols != 32) ||
+        (C + cols - 1) / cols > 65535 || R > 256)
         return (int)hipErrorInvalidValue;
     DeltaArgs p{q, ldq, k, ldk, v, ldv, g, ldg, b, ldb, out, ldo, state, slot_stride, seg_start, state_slots, R, C, share, heads, q_scale};
-    if (cols == 4) return launch_delta_cols<4>(p, segments, stream);
-    if (cols == 8) return launch_delta_cols<8>(p, segments, stream);
-    return launch_delta_cols<16>(p, segments, stream);
+    if (cols == 8) return launch_delta_group<16>(p, segments, stream);
+    if (cols == 16) return launch_delta_group<8>(p, segments, stream);
+    return launch_delta_group<4>(p, segments, stream);
 }
 
 // ------------------------------------------------------------------------------------------------ unit vectors

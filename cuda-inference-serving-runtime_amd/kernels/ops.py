@@ -78,6 +78,7 @@ def _declare(h):
         "cisr_latent_keys": [p, i, i, p, p, i, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, i, i, f, i, p],
         "cisr_heads_product": [p, i, i, p, p, i, i, p, i, i, i, i, i, i, p],
         "cisr_gelu": [p, p, ll, i, i, p],
+        "cisr_gemm_bf16_heads": [p, i, i, p, p, i, i, p, i, i, i, i, i, i, p],
     }
     for name, args in sig.items():
         fn = getattr(h, name)
@@ -1032,6 +1033,11 @@ def heads_product(a, a_head, w, out, out_head, gate=None):
     gp, ldg = (None, 0) if gate is None else _rows_of(gate, "gate", heads)
     if gate is not None and gate.shape[0] != rows:
         raise KernelError("heads_product: gates differ in rows")
+    if w.dtype == torch.bfloat16:
+        # the tiled matrix-core product, a launch for all heads (grid.y), the gate in its epilogue
+        _check(lib().cisr_gemm_bf16_heads(a.data_ptr(), a.stride(0), int(a_head), _dev(w, "w"), out.data_ptr(), out.stride(0),
+                                          int(out_head), gp, ldg, rows, n, k, heads, BF16, _stream()), "heads_product")
+        return out
     _check(lib().cisr_heads_product(a.data_ptr(), a.stride(0), int(a_head), _dev(w, "w"), out.data_ptr(), out.stride(0),
                                     int(out_head), gp, ldg, rows, heads, n, k, _storage(w, "w"), _stream()), "heads_product")
     return out
@@ -1239,6 +1245,15 @@ def unit_heads(x, heads, dim, scale=1.0, eps=1e-6):
     return x
 
 
+def delta_columns(segments, heads, cols):
+    """Columns of the state that one wave of the delta rule owns (32, 16 or 8): wide tiles read and write the state in
+    long runs (steps of many single tokens), narrow ones make more waves of the same head, until the launch has about
+    a wave for every SIMD of the GPU (a prompt's one segment is walked in order by every wave)."""
+    for width in (32, 16, 8):
+        if segments * heads * -(-cols // width) >= 1024 or width == 8:
+            return width
+
+
 def delta_scan(q, k, v, decay, write, out, state, seg_start, state_slots, heads, rows_of_state, cols_of_state, share=1,
                q_scale=1.0, columns=None):
     """Per segment and head, over the segment's rows in order: S <- g S; u = sigmoid(b) (v - S^T k); S <- S + k u^T;
@@ -1260,9 +1275,9 @@ def delta_scan(q, k, v, decay, write, out, state, seg_start, state_slots, heads,
         raise KernelError("delta_scan: operands differ in rows")
     if state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < heads * R * Cc or not state.is_cuda:
         raise KernelError("delta_scan: the state must be float [slots, >= heads * R * C]")
-    cols = int(columns or scan_columns(segments, heads, Cc))
-    while columns is None and cols > 4 and -(-R // (128 // cols)) > 16:
-        cols //= 2
+    cols = int(columns or delta_columns(segments, heads, Cc))
+    while columns is None and cols > 8 and -(-R // (128 // cols)) > 32:
+        cols //= 2         # (at most 32 rows of its two columns a lane)
     _check(_rec().cisr_delta_scan(qp, ldq, kp, ldk, vp, ldv, gp, ldg, bp, ldb, op, ldo, state.data_ptr(), state.stride(0),
                                   _dev(seg_start, "seg_start", torch.int32, (segments + 1,)),
                                   _dev(state_slots, "state_slots", torch.int32, (segments,)), segments, heads, R, Cc,

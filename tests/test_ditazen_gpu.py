@@ -159,7 +159,7 @@ def test_unit_vectors_a_head():
     assert (got[:, :4] == x[:, :4].astype(np.float32)).all()
 
 
-@pytest.mark.parametrize("heads, share, R, C, columns", [(3, 1, 16, 24, None), (4, 2, 40, 8, 4), (6, 3, 20, 16, 8), (4, 4, 12, 8, 16),
+@pytest.mark.parametrize("heads, share, R, C, columns", [(3, 1, 16, 24, None), (4, 2, 40, 8, 8), (6, 3, 20, 16, 32), (4, 4, 12, 8, 16), (2, 1, 256, 12, None), (1, 1, 128, 40, 32),
                                                          (1, 1, 5, 12, None), (2, 2, 130, 70, 16), (5, 1, 1, 3, None)])
 def test_delta_rule_over_segments_with_states_carried_and_slots_used_again(heads, share, R, C, columns):
     """Three segments of unequal length in one launch, then their continuations (one of them a single token) in another
