@@ -77,4 +77,20 @@ __device__ __forceinline__ float gated_activation(float g, float u, const GateLa
     return g / (1.0f + expf(-g)) * u;
 }
 
+// An ungated activation, the epilogue of a product that feeds a feed-forward's second matrix:
+//   1: z Phi(z), the gelu with the error function     2: its tanh form 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))
+enum { ACT_NONE = 0, ACT_GELU = 1, ACT_GELU_TANH = 2 };
+
+__device__ __forceinline__ float unary_activation(float z, int act) {
+    if (act == ACT_GELU) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
+    return 0.5f * z * (1.0f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
+}
+
+// as the epilogue of a product: the sum is rounded to the output's type first, as the path of two kernels does
+template <typename TC>
+__device__ __forceinline__ float activated(float v, int act) {
+    if (sizeof(TC) == 2) v = bf16_to_f32(f32_to_bf16(v));
+    return unary_activation(v, act);
+}
+
 #define CISR_LAUNCH_CHECK() ((int)hipGetLastError())

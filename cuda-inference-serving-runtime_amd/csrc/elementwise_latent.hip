@@ -200,16 +200,11 @@ extern "C" int cisr_heads_product(const void* a, int lda, int a_head, const void
 }
 
 // ------------------------------------------------------------------------------------------------ activation
-// kind 0: z Phi(z) with the error function; kind 1: 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))
-__device__ __forceinline__ float gelu_of(float z, int kind) {
-    if (kind == 0) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
-    return 0.5f * z * (1.0f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
-}
-
+// kind 0: the form with the error function; kind 1: the tanh form (unary_activation of common.h)
 template <typename T>
 __global__ void __launch_bounds__(256) gelu_kernel(const T* __restrict__ x, T* __restrict__ out, size_t n, int kind) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < n) store_f32(out + i, gelu_of(load_f32(x + i), kind));
+    if (i < n) store_f32(out + i, unary_activation(load_f32(x + i), kind == 0 ? ACT_GELU : ACT_GELU_TANH));
 }
 
 extern "C" int cisr_gelu(const void* x, void* out, long long n, int kind, int dtype, hipStream_t stream) {

@@ -128,8 +128,9 @@ __host__ __device__ inline int patch_side(int tiles) {
 // with gate and up of one output element in its registers and writes silu(gate) * up (both rounded to
 // bf16 first, as the two-kernel path does); a block then covers BN/2 output columns.
 // A batch of products in one launch (grid.y of them): product h reads A + h a, W + h w and writes C + h c (elements);
-// with `gate`, row m of product h is multiplied by sigmoid(gate[m * ldg + h]).  Zeros: one product, no gate.
-struct HeadBatch { long long a, w, c; const float* gate; int ldg; };
+// with `gate`, row m of product h is multiplied by sigmoid(gate[m * ldg + h]); with `act` (ACT_*, no residual) an ungated
+// activation is applied before the store.  Zeros: one product, no gate, no activation.
+struct HeadBatch { long long a, w, c; const float* gate; int ldg; int act; };
 
 template <int TM, int TN, int BK, typename TC, bool VEC, bool SWIGLU = false, int WM = 2>
 __global__ void __launch_bounds__(WM * 128)
@@ -303,7 +304,7 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int m = m0 + wm * TM * 16 + i * 16 + g * 4 + e;
-                if (m < M) store_f32(C + (size_t)m * ldc + n, acc[i][j][e]);
+                if (m < M) store_f32(C + (size_t)m * ldc + n, heads.act ? activated<TC>(acc[i][j][e], heads.act) : acc[i][j][e]);
             }
         }
     }
@@ -424,7 +425,7 @@ extern "C" int cisr_gemm_bf16_heads(const void* A, int lda, int a_head, const vo
     if (M <= 0 || N <= 0 || heads <= 0) return 0;
     if (K <= 0) return (int)hipErrorInvalidValue;
     const bf16_t* a = (const bf16_t*)A; const bf16_t* w = (const bf16_t*)W;
-    const HeadBatch batch{a_head, (long long)N * K, c_head, gate, ldg};
+    const HeadBatch batch{a_head, (long long)N * K, c_head, gate, ldg, ACT_NONE};
     auto blocks = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn) * heads; };
     int tile;
     if (M <= 32) tile = 122;
@@ -438,6 +439,30 @@ extern "C" int cisr_gemm_bf16_heads(const void* A, int lda, int a_head, const vo
         HEADS_TILE(1, 2, 2) HEADS_TILE(2, 2, 2) HEADS_TILE(4, 2, 2) HEADS_TILE(4, 4, 2)
     }
 #undef HEADS_TILE
+    return (int)hipErrorInvalidValue;
+}
+
+// C = act(A . W^T) with an ungated activation (ACT_GELU, ACT_GELU_TANH) as the epilogue; the tile is picked as for the
+// plain product.
+extern "C" int cisr_gemm_bf16_act(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N, int K,
+                                  int out_dtype, int act, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (K <= 0 || (act != ACT_GELU && act != ACT_GELU_TANH)) return (int)hipErrorInvalidValue;
+    const bf16_t* a = (const bf16_t*)A; const bf16_t* w = (const bf16_t*)W;
+    const HeadBatch batch{0, 0, 0, nullptr, 0, act};
+    auto blocks = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+    int tile;
+    if (M <= 32) tile = 122;
+    else if (blocks(128, 128) >= 512) tile = 442;
+    else if (blocks(128, 64) >= 512) tile = 422;
+    else if (blocks(64, 64) < 256) tile = 122;
+    else tile = 222;
+#define ACT_TILE(TM, TN, WM) \
+    case TM * 100 + TN * 10 + WM: return launch_bf16<TM, TN, 64, WM>(a, lda, w, ldw, C, ldc, nullptr, 0, M, N, K, out_dtype, stream, batch, 1);
+    switch (tile) {
+        ACT_TILE(1, 2, 2) ACT_TILE(2, 2, 2) ACT_TILE(4, 2, 2) ACT_TILE(4, 4, 2)
+    }
+#undef ACT_TILE
     return (int)hipErrorInvalidValue;
 }
 

@@ -14,6 +14,7 @@ struct SkinnyArgs {
     int M, N, K;
     int dual_off;                      // EPI_SWIGLU
     GateLaw law;                       // EPI_SWIGLU: the activation's law (zeros: silu(g) u)
+    int act;                           // EPI_STORE without a residual: an ungated activation before the store (ACT_*)
     // NORM
     const float* norm_w; float eps; const int* rows;
     // EPI_ROPE

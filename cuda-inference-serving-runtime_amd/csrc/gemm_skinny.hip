@@ -65,12 +65,18 @@ static int launch_narrow(const SkinnyArgs& a, int units, bool norm, int epi, int
 // [*, K] (rows picked by `rows` if given).  dual_off > 0 selects SwiGLU over two blocks of N rows of W.
 static int skinny_entry(const void* A, int lda, const void* W, int ldw, void* C, int ldc, const float* R,
                         int ldr, int M, int N, int K, int out_dtype, int dual_off, const float* norm_w,
-                        float eps, const int* rows, GateLaw law, hipStream_t stream);
+                        float eps, const int* rows, GateLaw law, hipStream_t stream, int act);
 
 extern "C" int cisr_gemm_skinny_bf16(const void* A, int lda, const void* W, int ldw, void* C, int ldc, const float* R,
                                      int ldr, int M, int N, int K, int out_dtype, int dual_off, const float* norm_w,
                                      float eps, const int* rows, hipStream_t stream) {
-    return skinny_entry(A, lda, W, ldw, C, ldc, R, ldr, M, N, K, out_dtype, dual_off, norm_w, eps, rows, GateLaw{}, stream);
+    return skinny_entry(A, lda, W, ldw, C, ldc, R, ldr, M, N, K, out_dtype, dual_off, norm_w, eps, rows, GateLaw{}, stream, ACT_NONE);
+}
+
+// C = act(A . W^T): the same product with an ungated activation (ACT_GELU, ACT_GELU_TANH) before the store.
+extern "C" int cisr_gemm_skinny_bf16_act(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N, int K,
+                                         int out_dtype, int act, hipStream_t stream) {
+    return skinny_entry(A, lda, W, ldw, C, ldc, nullptr, 0, M, N, K, out_dtype, 0, nullptr, 0.f, nullptr, GateLaw{}, stream, act);
 }
 
 // The product over [gate; up] (dual_off > 0) with the gated activation's law given: see GateLaw.
@@ -78,19 +84,20 @@ extern "C" int cisr_gemm_skinny_bf16_gated(const void* A, int lda, const void* W
                                            int dual_off, float limit, float slope, float shift, hipStream_t stream) {
     if (dual_off <= 0) return (int)hipErrorInvalidValue;
     return skinny_entry(A, lda, W, ldw, C, ldc, nullptr, 0, M, N, K, DT_BF16, dual_off, nullptr, 0.f, nullptr,
-                        GateLaw{limit, slope, shift}, stream);
+                        GateLaw{limit, slope, shift}, stream, ACT_NONE);
 }
 
 static int skinny_entry(const void* A, int lda, const void* W, int ldw, void* C, int ldc, const float* R,
                         int ldr, int M, int N, int K, int out_dtype, int dual_off, const float* norm_w,
-                        float eps, const int* rows, GateLaw law, hipStream_t stream) {
+                        float eps, const int* rows, GateLaw law, hipStream_t stream, int act) {
     if (M <= 0 || N <= 0) return 0;
+    if (act < ACT_NONE || act > ACT_GELU_TANH || (act && (R || dual_off > 0))) return (int)hipErrorInvalidValue;
     if (M > 64 || K <= 0 || K % 8 || lda % 8 || ldw % 8 || !aligned16(A) || !aligned16(W) ||
         (R && out_dtype != DT_F32) || (norm_w && !aligned16(norm_w)) || (dual_off > 0 && (R || out_dtype != DT_BF16)))
         return (int)hipErrorInvalidValue;
     SkinnyArgs a = {};
     a.A = A; a.lda = lda; a.W = (const bf16_t*)W; a.ldw = ldw; a.C = C; a.ldc = ldc; a.R = R; a.ldr = ldr;
-    a.M = M; a.N = N; a.K = K; a.dual_off = dual_off; a.norm_w = norm_w; a.eps = eps; a.rows = rows; a.law = law;
+    a.M = M; a.N = N; a.K = K; a.dual_off = dual_off; a.norm_w = norm_w; a.eps = eps; a.rows = rows; a.law = law; a.act = act;
     const int epi = dual_off > 0 ? EPI_SWIGLU : EPI_STORE;
     if (cisr_gemv_ok(M, dual_off > 0 ? 2 * N : N, K)) return cisr_gemv_launch(a, N, norm_w != nullptr, epi, out_dtype, 0, stream);
     if (narrow_wanted(M, dual_off > 0 ? 2 * N : N, K, norm_w != nullptr)) return launch_narrow(a, (N + 3) / 4, norm_w != nullptr, epi, out_dtype, stream);

@@ -320,6 +320,7 @@ gemv_kernel(SkinnyArgs p, int units, int per_wave) {
         float v0 = v[0] * scale;
         if (EPI == EPI_STORE) {
             if (p.R) v0 += resid;
+            if (p.act) v0 = activated<TC>(v0, p.act);
             store_f32((TC*)p.C + (size_t)m * p.ldc + u, v0);
         } else if (EPI == EPI_SWIGLU) {
             const float v1 = v[R - 1] * scale;

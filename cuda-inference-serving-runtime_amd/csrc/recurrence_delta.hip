@@ -45,13 +45,16 @@ __device__ __forceinline__ float group_sum(float x) {
 }
 
 // A wave a (segment, head, tile of COLS = 128 / NG columns); NG neighbouring lanes share two neighbouring columns, and
-// lane l of them owns the rows l + NG i, i < RPT, of the state in registers.  Rows of a segment are walked in order,
-// GROUP at a time through LDS, the next group's loads in flight while this one is walked; inside a group the next
-// row's operands are read from LDS while this row's sums meet.
+// lane l of them owns the rows l RPT + i, i < RPT, of the state in registers.  Rows of a segment are walked in order,
+// GROUP at a time through LDS, the next group's loads in flight while this one is walked.  In LDS a lane's RPT
+// coordinates of q and of k lie side by side (one wide read each), the lanes' runs PAD floats apart so that the reads of
+// the sixteen lanes of a row fall into different banks.
 template <int NG, int RPT>
 __global__ void __launch_bounds__(64) delta_scan_kernel(DeltaArgs p) {
     constexpr int LPG = WAVE / NG, COLS = 2 * LPG, GROUP = DELTA_GROUP_OF(RPT), RP = NG * RPT;
-    __shared__ float sq[GROUP * RP], sk[GROUP * RP], sg[GROUP], sb[GROUP], sv[GROUP * COLS];
+    constexpr int PAD = RPT >= 4 ? 4 : 2, RUN = RPT + PAD, RPS = NG * RUN;     // floats of a lane's run, of a row in LDS
+    __shared__ __attribute__((aligned(16))) float sq[GROUP * RPS], sk[GROUP * RPS];
+    __shared__ float sg[GROUP], sb[GROUP], sv[GROUP * COLS];
     const int seg = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
     const int t0 = p.seg_start[seg], t1 = p.seg_start[seg + 1];
     if (t1 <= t0) return;
@@ -64,9 +67,9 @@ __global__ void __launch_bounds__(64) delta_scan_kernel(DeltaArgs p) {
     float S0[RPT], S1[RPT];
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
-        const bool in = rg + NG * i < R;
-        S0[i] = in ? state[(size_t)(rg + NG * i) * C + c0] : 0.f;
-        S1[i] = in ? state[(size_t)(rg + NG * i) * C + c1] : 0.f;
+        const bool in = rg * RPT + i < R;
+        S0[i] = in ? state[(size_t)(rg * RPT + i) * C + c0] : 0.f;
+        S1[i] = in ? state[(size_t)(rg * RPT + i) * C + c1] : 0.f;
     }
     const float* qh = p.q + (size_t)(head / p.share) * R;
     const float* kh = p.k + (size_t)(head / p.share) * R;
@@ -102,8 +105,9 @@ __global__ void __launch_bounds__(64) delta_scan_kernel(DeltaArgs p) {
         __syncthreads();                                   // (the walk before is over: LDS may be written)
 #pragma unroll
         for (int j = 0; j < PF; ++j) {
-            sk[lane + WAVE * j] = fk[j];
-            sq[lane + WAVE * j] = fq[j];
+            const int idx = lane + WAVE * j, tt = idx / RP, r = idx % RP;
+            sk[tt * RPS + (r / RPT) * RUN + r % RPT] = fk[j];
+            sq[tt * RPS + (r / RPT) * RUN + r % RPT] = fq[j];
         }
 #pragma unroll
         for (int j = 0; j < PV; ++j)
@@ -114,21 +118,17 @@ __global__ void __launch_bounds__(64) delta_scan_kernel(DeltaArgs p) {
         }
         __syncthreads();
         if (tb + GROUP < t1) fetch(tb + GROUP);
-        float kc[RPT], qc[RPT], v0, v1, g, beta;
-        auto take = [&](int tt) {
+#pragma unroll
+        for (int tt = 0; tt < GROUP; ++tt) {
+            if (tt >= n) break;                            // (uniform over the wave)
+            float kc[RPT], qc[RPT];
 #pragma unroll
             for (int i = 0; i < RPT; ++i) {
-                kc[i] = sk[tt * RP + rg + NG * i];
-                qc[i] = sq[tt * RP + rg + NG * i];
+                kc[i] = sk[tt * RPS + rg * RUN + i];
+                qc[i] = sq[tt * RPS + rg * RUN + i];
             }
-            v0 = sv[tt * COLS + 2 * pair];
-            v1 = sv[tt * COLS + 2 * pair + 1];
-            g = sg[tt];
-            beta = sb[tt];
-        };
-        take(0);
-#pragma unroll 1
-        for (int tt = 0; tt < n; ++tt) {
+            const float v0 = sv[tt * COLS + 2 * pair], v1 = sv[tt * COLS + 2 * pair + 1];
+            const float g = sg[tt], beta = sb[tt];
             float sk0 = 0.f, sk1 = 0.f, sq0 = 0.f, sq1 = 0.f, kq = 0.f;
 #pragma unroll
             for (int i = 0; i < RPT; ++i) {
@@ -138,34 +138,29 @@ __global__ void __launch_bounds__(64) delta_scan_kernel(DeltaArgs p) {
                 sq1 += S1[i] * qc[i];
                 kq += kc[i] * qc[i];
             }
-            float kn[RPT];
-#pragma unroll
-            for (int i = 0; i < RPT; ++i) kn[i] = kc[i];
-            const float gn = g, bn = beta, w0 = v0, w1 = v1;
-            if (tt + 1 < n) take(tt + 1);                  // the next row's operands are on their way while the sums meet
             sk0 = group_sum<NG>(sk0);
             sk1 = group_sum<NG>(sk1);
             sq0 = group_sum<NG>(sq0);
             sq1 = group_sum<NG>(sq1);
             kq = group_sum<NG>(kq);
-            const float u0 = bn * (w0 - gn * sk0), u1 = bn * (w1 - gn * sk1);
+            const float u0 = beta * (v0 - g * sk0), u1 = beta * (v1 - g * sk1);
 #pragma unroll
             for (int i = 0; i < RPT; ++i) {
-                S0[i] = gn * S0[i] + kn[i] * u0;
-                S1[i] = gn * S1[i] + kn[i] * u1;
+                S0[i] = g * S0[i] + kc[i] * u0;
+                S1[i] = g * S1[i] + kc[i] * u1;
             }
             if (rg == 0) {
                 float* o = p.out + (size_t)(tb + tt) * p.ldo + (size_t)head * C;
-                if (ok0) o[c] = (gn * sq0 + kq * u0) * p.q_scale;
-                if (ok1) o[c + 1] = (gn * sq1 + kq * u1) * p.q_scale;
+                if (ok0) o[c] = (g * sq0 + kq * u0) * p.q_scale;
+                if (ok1) o[c + 1] = (g * sq1 + kq * u1) * p.q_scale;
             }
         }
     }
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
-        if (rg + NG * i >= R) continue;
-        if (ok0) state[(size_t)(rg + NG * i) * C + c] = S0[i];
-        if (ok1) state[(size_t)(rg + NG * i) * C + c + 1] = S1[i];
+        if (rg * RPT + i >= R) continue;
+        if (ok0) state[(size_t)(rg * RPT + i) * C + c] = S0[i];
+        if (ok1) state[(size_t)(rg * RPT + i) * C + c + 1] = S1[i];
     }
 }
 

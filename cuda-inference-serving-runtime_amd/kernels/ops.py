@@ -79,6 +79,8 @@ def _declare(h):
         "cisr_heads_product": [p, i, i, p, p, i, i, p, i, i, i, i, i, i, p],
         "cisr_gelu": [p, p, ll, i, i, p],
         "cisr_gemm_bf16_heads": [p, i, i, p, p, i, i, p, i, i, i, i, i, i, p],
+        "cisr_gemm_skinny_bf16_act": [p, i, p, i, p, i, i, i, i, i, i, p],
+        "cisr_gemm_bf16_act": [p, i, p, i, p, i, i, i, i, i, i, p],
     }
     for name, args in sig.items():
         fn = getattr(h, name)
@@ -1044,6 +1046,31 @@ def heads_product(a, a_head, w, out, out_head, gate=None):
 
 
 GELU_KINDS = {"gelu": 0, "gelu_erf": 0, "gelu_tanh": 1}
+
+
+def gemm_gelu(a, w, out, kind="gelu", scratch=None, product=None):
+    """out[M, N] = gelu(a . w^T), out of the operands' dtype.  bf16 products of this repository's own kernels (few rows
+    against weights that the wide kernel does not take; many rows against weights that the library does not take) apply
+    the activation as their epilogue; the others run the product into `product` ([M, N], a buffer of the caller's) and
+    the activation as a kernel after it, as the gated feed-forwards do beside the library's product."""
+    if kind not in GELU_KINDS:
+        raise KernelError(f"gelu: unknown form {kind!r}")
+    m, k = a.shape
+    n = w.shape[0]
+    fused = (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and tuple(out.shape) == (m, n)
+             and w.shape[1] == k and a.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1 and not library_ok(m, w))
+    act = 1 + GELU_KINDS[kind]
+    if fused and m <= SKINNY_ROWS and _skinny_ok(a, w) and not wide_ok(m, w):
+        _check(lib().cisr_gemm_skinny_bf16_act(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0),
+                                               m, n, k, BF16, act, _stream()), "gemm_gelu")
+        return out
+    if fused and m > SKINNY_ROWS:
+        _check(lib().cisr_gemm_bf16_act(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0),
+                                        m, n, k, BF16, act, _stream()), "gemm_gelu")
+        return out
+    if product is None:
+        raise KernelError("gemm_gelu: this product needs a buffer for its result before the activation")
+    return gelu(gemm(a, w, product, scratch=scratch), out, kind)
 
 
 def gelu(x, out, kind="gelu"):

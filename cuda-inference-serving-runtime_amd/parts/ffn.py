@@ -114,8 +114,9 @@ class DenseMLP(FeedForward):
 
     def _activations(self, h, ctx):
         T = h.shape[0]
-        up = ops.gemm(h, self.w_up, ctx.buffer("ffn.up", (T, self.intermediate), ctx.dtype), scratch=ctx.scratch)
-        return ops.gelu(up, ctx.buffer("ffn.act", (T, self.intermediate), ctx.dtype), self.activation)
+        # the activation is the epilogue of the product where a kernel of this repository runs it
+        return ops.gemm_gelu(h, self.w_up, ctx.buffer("ffn.act", (T, self.intermediate), ctx.dtype), self.activation, scratch=ctx.scratch,
+                             product=ctx.buffer("ffn.up", (T, self.intermediate), ctx.dtype))
 
     def output(self, h, ctx):
         """The feed-forward's result, float [T, hidden], without the residual sum."""

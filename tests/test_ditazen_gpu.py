@@ -81,6 +81,27 @@ def test_gelu(form, dtype):
     close(got, want, 2e-6 if dtype == "float32" else 5e-3)
 
 
+@pytest.mark.parametrize("form", ["gelu", "gelu_tanh"])
+@pytest.mark.parametrize("rows", [1, 3, 16, 40, 100, 300])
+@pytest.mark.parametrize("inner, width", [(64, 48), (1024, 4096), (100, 52)])
+def test_gelu_as_the_epilogue_of_the_product_before_it(rows, inner, width, form):
+    """Every kernel that takes the product (matrix-vector, narrow, skinny, tiled; with other sizes the product and the
+    activation as two kernels) gives gelu of the product rounded to bfloat16."""
+    from runtime.kernels import ops
+    rng = np.random.default_rng(rows + inner)
+    a = dev(rng.standard_normal((rows, inner)), torch.bfloat16)
+    w = dev(rng.standard_normal((width, inner)) / np.sqrt(inner) * 2.0, torch.bfloat16)
+    out = torch.empty(rows, width, device=DEV, dtype=torch.bfloat16)
+    ops.gemm_gelu(a, w, out, form, product=torch.empty(rows, width, device=DEV, dtype=torch.bfloat16))
+    want = P.ACTIVATIONS[form](rounded(host(a) @ host(w).T))
+    err = np.abs(host(out) - want).max() / np.abs(want).max()
+    assert err < 1e-2, f"differs by {err:.3e}"
+    for dtype in (torch.float32,):
+        a32, w32 = a.float(), w.float()
+        out32 = ops.gemm_gelu(a32, w32, torch.empty(rows, width, device=DEV), form, product=torch.empty(rows, width, device=DEV))
+        close(host(out32), P.ACTIVATIONS[form](host(a) @ host(w).T), 1e-5)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads, dim, rot_dim, rot, rank, interleaved", [(3, 16, 8, 8, 40, False), (2, 24, 16, 16, 48, True),
                                                                            (1, 10, 6, 4, 20, True), (5, 8, 12, 6, 9, False)])
