@@ -37,13 +37,74 @@ layernorm_kernel(const float* __restrict__ x, const float* __restrict__ w, const
     for (int i = threadIdx.x; i < dim; i += 256) store_f32(o + i, (xr[i] - mean) * inv * w[i] + (b ? b[i] : 0.f));
 }
 
+// Rows of a multiple of four floats, at most 256 CH of them, 16-byte aligned: one wave a row, the row in registers (CH
+// words of four floats a lane), no barrier; the statistics meet over the lanes.
+template <typename OUT, int CH>
+__global__ void __launch_bounds__(256)
+layernorm_wave_kernel(const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ b,
+                      OUT* __restrict__ out, const int* __restrict__ rows, int n_out, int dim, float eps) {
+    typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+    const int r = blockIdx.x * 4 + threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    if (r >= n_out) return;
+    const f32x4_t* xr = (const f32x4_t*)(x + (size_t)(rows ? rows[r] : r) * dim);
+    const int words = dim / 4;
+    f32x4_t v[CH];
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+        const int at = lane + WAVE * i;
+        v[i] = at < words ? xr[at] : (f32x4_t){0.f, 0.f, 0.f, 0.f};
+        s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+    }
+    const float mean = wave_sum(s) / dim;
+    float q = 0.f;
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+        if (lane + WAVE * i >= words) continue;
+        v[i].x -= mean; v[i].y -= mean; v[i].z -= mean; v[i].w -= mean;
+        q += (v[i].x * v[i].x + v[i].y * v[i].y) + (v[i].z * v[i].z + v[i].w * v[i].w);
+    }
+    const float inv = rsqrtf(wave_sum(q) / dim + eps);
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+        const int at = lane + WAVE * i;
+        if (at >= words) continue;
+        const f32x4_t ww = ((const f32x4_t*)w)[at];
+        const f32x4_t bb = b ? ((const f32x4_t*)b)[at] : (f32x4_t){0.f, 0.f, 0.f, 0.f};
+        const f32x4_t y = {v[i].x * inv * ww.x + bb.x, v[i].y * inv * ww.y + bb.y, v[i].z * inv * ww.z + bb.z, v[i].w * inv * ww.w + bb.w};
+        if (sizeof(OUT) == 4) {
+            ((f32x4_t*)((float*)out + (size_t)r * dim))[at] = y;
+        } else {
+            typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
+            ((u32x2_t*)((bf16_t*)out + (size_t)r * dim))[at] = (u32x2_t){pack_bf16x2(y.x, y.y), pack_bf16x2(y.z, y.w)};
+        }
+    }
+}
+
+template <typename OUT>
+static int launch_layernorm(const float* x, const float* w, const float* b, OUT* out, const int* rows, int n_out, int dim,
+                            float eps, hipStream_t stream) {
+    const bool aligned = dim % 4 == 0 && ((uintptr_t)x) % 16 == 0 && ((uintptr_t)w) % 16 == 0 && (!b || ((uintptr_t)b) % 16 == 0) &&
+                         ((uintptr_t)out) % 16 == 0;
+    const int per_lane = (dim / 4 + WAVE - 1) / WAVE;
+    const unsigned blocks = (unsigned)((n_out + 3) / 4);
+#define LN_WAVE(CH) layernorm_wave_kernel<OUT, CH><<<blocks, 256, 0, stream>>>(x, w, b, out, rows, n_out, dim, eps)
+    if (aligned && per_lane <= 1) LN_WAVE(1);
+    else if (aligned && per_lane <= 2) LN_WAVE(2);
+    else if (aligned && per_lane <= 4) LN_WAVE(4);
+    else if (aligned && per_lane <= 8) LN_WAVE(8);
+    else if (aligned && per_lane <= 16) LN_WAVE(16);
+    else layernorm_kernel<OUT><<<n_out, 256, 0, stream>>>(x, w, b, out, rows, dim, eps);
+#undef LN_WAVE
+    return CISR_LAUNCH_CHECK();
+}
+
 extern "C" int cisr_layernorm(const float* x, const float* w, const float* b, void* out, const int* rows, int n_out,
                               int dim, float eps, int out_dtype, hipStream_t stream) {
     if (n_out <= 0) return 0;
     if (dim <= 0) return (int)hipErrorInvalidValue;
-    if (out_dtype == DT_F32) layernorm_kernel<float><<<n_out, 256, 0, stream>>>(x, w, b, (float*)out, rows, dim, eps);
-    else layernorm_kernel<bf16_t><<<n_out, 256, 0, stream>>>(x, w, b, (bf16_t*)out, rows, dim, eps);
-    return CISR_LAUNCH_CHECK();
+    if (out_dtype == DT_F32) return launch_layernorm<float>(x, w, b, (float*)out, rows, n_out, dim, eps, stream);
+    return launch_layernorm<bf16_t>(x, w, b, (bf16_t*)out, rows, n_out, dim, eps, stream);
 }
 
 // ------------------------------------------------------------------------------------------------ rms of a slice

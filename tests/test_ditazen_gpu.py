@@ -52,7 +52,7 @@ def rounded(a):
 
 # -- mechanisms alone -----------------------------------------------------------------------------------------------------
 
-@pytest.mark.parametrize("dim", [64, 100, 1, 777])
+@pytest.mark.parametrize("dim", [64, 100, 1, 777, 2048, 4100])
 def test_centred_norm_and_the_norm_of_a_slice(dim):
     from runtime.kernels import ops
     rng = np.random.default_rng(dim)
