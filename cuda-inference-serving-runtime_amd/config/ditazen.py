@@ -67,8 +67,8 @@ class LatentSpec:
         rot = RotarySpec.from_dict(rot, where + ".rot")
         if rot.dims > rot_dim:
             raise ConfigError(f"{where}: rot.dims {rot.dims} exceeds rot_dim {rot_dim}")
-        if kv_rank + rot_dim > 256:
-            raise ConfigError(f"{where}: kv_rank + rot_dim of at most 256 is supported")
+        if kv_rank + rot_dim > 640:
+            raise ConfigError(f"{where}: kv_rank + rot_dim of at most 640 is supported")
         q_rank = raw.get("q_rank") if second else None
         if q_rank is not None:
             _positive_ints((q_rank,), where + ".q_rank")

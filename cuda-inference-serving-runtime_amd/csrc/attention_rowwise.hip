@@ -5,14 +5,15 @@
 // tensor (reference: docs/ARCHITECTURE.md:20-21, kernels/execution.cu:48-79).
 // This kernel is exact float arithmetic on float or bf16 storage and serves as
 // the 32-bit path and as the general fallback; it takes any even head size up
-// to 256, any page size, any head grouping.
+// to 640, any page size, any head grouping.
 //
 // Within a block of 64 keys each lane scores one key (q is broadcast from LDS),
 // the wave reduces the running maximum and denominator once per 64 keys, then
 // each lane accumulates its own output coordinates over the 64 keys.
 #include "common.h"
 
-#define MAX_HEAD_DIM 256
+#define MAX_HEAD_DIM 640
+#define MAX_COORDS (MAX_HEAD_DIM / WAVE)     // output coordinates a lane
 
 template <typename T>
 __global__ void __launch_bounds__(64)
@@ -29,9 +30,11 @@ attn_rowwise_kernel(const T* __restrict__ q, int q_row_stride, const T* __restri
     const int row = blockIdx.x, head = blockIdx.y, split = blockIdx.z, lane = threadIdx.x;
     const int kvh = head / (heads / kv_heads);
     const int seg = seg_of_row[row];
-    const int ncoord = (dim + WAVE - 1) / WAVE;  // at most 4
+    const int ncoord = (dim + WAVE - 1) / WAVE;  // at most MAX_COORDS
 
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    float acc[MAX_COORDS];
+#pragma unroll
+    for (int c = 0; c < MAX_COORDS; ++c) acc[c] = 0.f;
     float m = -INFINITY, l = 0.f;
     int begin = 0, end = 0;
     if (seg >= 0) {
@@ -72,7 +75,7 @@ attn_rowwise_kernel(const T* __restrict__ q, int q_row_stride, const T* __restri
             __syncthreads();
             const int nvalid = min(WAVE, end - base);
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
+            for (int c = 0; c < MAX_COORDS; ++c) {
                 if (c < ncoord) {
                     const int d = lane + c * WAVE;
                     float a = acc[c] * alpha;
@@ -87,14 +90,14 @@ attn_rowwise_kernel(const T* __restrict__ q, int q_row_stride, const T* __restri
     if (splits == 1) {
         T* o = out + ((size_t)row * heads + head) * dim;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
+        for (int c = 0; c < MAX_COORDS; ++c) {
             const int d = lane + c * WAVE;
             if (c < ncoord && d < dim) store_f32(o + d, acc[c] * inv);
         }
     } else {
         const size_t part = ((size_t)row * heads + head) * splits + split;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
+        for (int c = 0; c < MAX_COORDS; ++c) {
             const int d = lane + c * WAVE;
             if (c < ncoord && d < dim) part_o[part * dim + d] = acc[c] * inv;
         }

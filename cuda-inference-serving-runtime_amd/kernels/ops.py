@@ -300,14 +300,17 @@ def f32_to_bf16(x, out):
     return out
 
 
+ROWWISE_MAX_HEAD = 640     # the row-wise attention kernel's largest head (the matrix-core kernels stop at 256)
+
+
 def attention_rowwise(q, q_row_stride, kcache, vcache, tables, seg_of_row, positions, out, heads, kv_heads, dim,
                       page_size, window, scale, splits=1, workspace=None):
     """Each row attends to its request's cached keys lo..position.  q is a view
     into a row-major buffer with `q_row_stride` elements per row; out [T, heads*dim]."""
     rows = out.shape[0]
     dt = _storage(out, "out")
-    if dim % 2 or dim > 256:
-        raise KernelError(f"attention: head size {dim} must be even and at most 256")
+    if dim % 2 or dim > ROWWISE_MAX_HEAD:
+        raise KernelError(f"attention: head size {dim} must be even and at most {ROWWISE_MAX_HEAD}")
     if heads % kv_heads:
         raise KernelError(f"attention: {heads} query heads do not divide into {kv_heads} key heads")
     pages = kcache.shape[0]

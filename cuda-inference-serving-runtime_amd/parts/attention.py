@@ -222,7 +222,8 @@ class LatentAttention(Mixer):
     is that of `heads` query heads [q'_j | rot(qr_j)] over ONE key head [c | kr] and one value head [c] of
     pad = rank + rot_dim coordinates (rounded up to 8, the rest zero), which the framework's paged attention kernels
     run as they are; the weighted sum of latents then goes through Wuv_j.  The pages therefore hold what the design
-    says must be kept, c and kr, and nothing a head.  `position` turns the first `position.rotary_dim` of the rot_dim
+    says must be kept, c and kr, and nothing a head.  Up to 256 coordinates the matrix-core kernels serve (bfloat16); a
+    larger latent (up to 640 with its turning part) runs the exact row-wise kernel in both dtypes.  `position` turns the first `position.rotary_dim` of the rot_dim
     coordinates.  `names`: the tensors' names under `name`."""
 
     NAMES = {"q": "q", "dq": "dq", "dq_norm": "dq.norm", "uq": "uq", "dkv": "dkv", "dkv_norm": "dkv.norm", "uk": "uk",
@@ -231,8 +232,8 @@ class LatentAttention(Mixer):
     def __init__(self, name, hidden, heads, dim, rot_dim, vdim, kv_rank, scale, eps, position, q_rank=None, window=None,
                  head_gate=True, names=None, tuning=None):
         self.pad = -(-(kv_rank + rot_dim) // 8) * 8
-        if self.pad > 256:
-            raise ValueError(f"a latent of {kv_rank} and {rot_dim} turning coordinates: at most 256 together")
+        if self.pad > ops.ROWWISE_MAX_HEAD:
+            raise ValueError(f"a latent of {kv_rank} and {rot_dim} turning coordinates: at most {ops.ROWWISE_MAX_HEAD} together")
         if not scale > 0:
             raise ValueError("the score scale must be positive")
         if position.rotary_dim > rot_dim:

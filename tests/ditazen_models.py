@@ -69,10 +69,16 @@ CONFIGS = {
     # sharp: one key carries a query, decays close to one (the weights' maker reads "sharp"); the window and the full
     # layer run twice
     "s": config(97, 48, 0.6, 1e-5, _S + [again(_S[0], 0), again(_S[2], 2)]),
+    # twenty heads over the one key head (more than the sixteen a wave's tile of the matrix-core kernels holds), and a
+    # latent too large for those kernels (it runs the row-wise kernel); a state of 256 rows
+    "w": config(61, 56, 0.8, 1e-5, [
+        latent(20, 8, 8, 8, 16, 0.3, rot(500.0, 8), 33, mlp(40)),
+        latent2(3, 8, 8, 16, 296, 16, 0.06, rot(3000.0, 8, (2.0, 64, 8.0, 2.0))),
+        delta(2, 1, 256, 8, 2)]),
     # no layer keeps pages: the cache manager has state slots only
     "d": config(53, 40, 1.0, 1e-5, [delta(4, 1, 8, 12, 2, mlp(48)), delta(3, 3, 20, 8, 5)]),
 }
-SEEDS = {"a": 21, "b": 22, "s": 23, "d": 24}
+SEEDS = {"a": 21, "b": 22, "s": 23, "d": 24, "w": 25}
 FILE_Q_RANK = 28       # the query latent of configuration "b", which config.json does not give
 
 

@@ -1252,7 +1252,7 @@ def test_page_copy(ops):
 def test_kernels_refuse_what_they_cannot_take(ops):
     from runtime.kernels.ops import KernelError
     with pytest.raises(KernelError, match="head size"):
-        run_rowwise(ops, rnd(1, 2, 258), rnd(1, 2, 4, 258), rnd(1, 2, 258, 4), torch.zeros(1, 1, dtype=torch.int32, device=DEV), [(0, 0)], 4)
+        run_rowwise(ops, rnd(1, 2, 642), rnd(1, 2, 4, 642), rnd(1, 2, 642, 4), torch.zeros(1, 1, dtype=torch.int32, device=DEV), [(0, 0)], 4)
     with pytest.raises(KernelError, match="divide"):
         run_rowwise(ops, rnd(1, 3, 16), rnd(1, 2, 4, 16), rnd(1, 2, 16, 4), torch.zeros(1, 1, dtype=torch.int32, device=DEV), [(0, 0)], 4)
     with pytest.raises(KernelError, match="not supported"):   # the matrix-core kernel takes bf16, head sizes in steps of 8, pages of 8, 16, ... keys
