@@ -192,15 +192,20 @@ class DitazenConfig:
             raise ConfigError("config.json: norm.eps must be a number >= 0")
         limit = raw.get("max_positions", cls.max_positions)
         _positive_ints((limit,), "config.json max_positions")
-        typed = tuple(DitazenLayer.from_dict(layer, f"layers[{i}]") for i, layer in enumerate(layers))
+        typed = [DitazenLayer.from_dict(layer, f"layers[{i}]") for i, layer in enumerate(layers)]
         for i, layer in enumerate(typed):
-            j = layer.weights_of
+            j, seen = layer.weights_of, {i}
             if j is None:
                 continue
-            if j >= len(typed) or j == i or typed[j].weights_of is not None:
-                raise ConfigError(f"layers[{i}]: weights_of {j} must name another layer that has tensors of its own")
+            while j is not None and j < len(typed) and j not in seen and typed[j].weights_of is not None:
+                seen.add(j)                   # (a layer that names a layer that names another: the one that has the tensors)
+                j = typed[j].weights_of
+            if j is None or j >= len(typed) or j in seen:
+                raise ConfigError(f"layers[{i}]: weights_of {layer.weights_of} must lead to another layer that has tensors of its own")
             if not layer.same_weights(typed[j]):
                 raise ConfigError(f"layers[{i}]: its entry differs from that of layer {j}, whose weights it uses")
+            typed[i] = DitazenLayer(layer.type, layer.latent, layer.delta, layer.mlp, j)
+        typed = tuple(typed)
         return cls(vocab, width, typed, float(norm["eps"]), float(raw.get("logit_scale", 1.0)), limit)
 
     def to_dict(self):

@@ -174,6 +174,20 @@ def test_config_errors_name_the_place():
             DitazenConfig.from_dict(raw)
 
 
+def test_a_layer_may_name_a_layer_that_names_the_one_with_the_tensors():
+    from runtime.config import DitazenConfig, ConfigError
+    from runtime.engine.loading import build_from_config_dict
+    raw = json.loads(json.dumps(CONFIGS["a"]))
+    raw["layers"].append({**json.loads(json.dumps(raw["layers"][3])), "weights_of": 3})      # layer 3 runs with layer 1's
+    cfg = DitazenConfig.from_dict(raw)
+    assert [layer.weights_of for layer in cfg.layers] == [None, None, None, 1, 0, 1]
+    _, _, model = build_from_config_dict(raw)
+    assert [entry.layer for entry in model.schedule] == [0, 1, 2, 1, 0, 1] and sorted(model.state_needs()) == [1, 3, 5]
+    raw["layers"][1]["weights_of"] = 5                                                        # a ring has no tensors at all
+    with pytest.raises(ConfigError, match=r"layers\[1\]"):
+        DitazenConfig.from_dict(raw)
+
+
 def test_rotary_tables_of_the_framework_follow_the_scaling():
     from runtime.parts import RotaryEmbedding
     rot = {"base": 50000.0, "dims": 16, "scaling": {"factor": 8.0, "original": 64, "fast": 16.0, "slow": 2.0}}
