@@ -453,3 +453,52 @@ def test_command_line_serves_the_design(folders, tmp_path):
     out = json.loads(proc.stdout)
     assert out["weights"] == "random-ditazen-tiny" and len(out["requests"][0]["generated"]) == 3
     assert out["runner"]["replays"] >= 1 and out["runner"]["cache"][0]["resident_pages"] == 0
+
+
+def random_config(seed):
+    """A configuration drawn at random: sizes, head counts, the order of the layers, windows, constants; some layers run
+    with earlier layers' weights."""
+    from ditazen_models import config, delta, latent, latent2, mlp, rot, again
+    rng = np.random.default_rng(seed)
+    pick = lambda *values: values[int(rng.integers(len(values)))]
+    layers = []
+    for _ in range(int(rng.integers(2, 6))):
+        kind = pick("latent_attention", "latent_attention_2", "delta")
+        ff = pick(None, mlp(int(rng.integers(3, 12)) * 8), mlp(int(rng.integers(20, 90)), pick(None, "gelu_tanh")))
+        if kind == "delta":
+            kv_heads = pick(1, 2, 3)
+            layers.append(delta(kv_heads * pick(1, 2, 4), kv_heads, pick(8, 12, 32, 40, 64), pick(8, 16, 24, 48), pick(1, 2, 4, 5), ff))
+            continue
+        rot_dim = pick(4, 8, 16, 32)
+        dims = pick(rot_dim, rot_dim, max(2, rot_dim // 2))
+        scaling = (pick(2.0, 4.0, 16.0), pick(16, 64, 256), pick(8.0, 32.0), pick(1.0, 2.0))
+        sizes = (pick(1, 2, 4, 5, 8), pick(8, 16, 24, 64), rot_dim, pick(8, 16, 40, 80), pick(16, 24, 64, 96, 128))
+        if kind == "latent_attention":
+            layers.append(latent(*sizes, float(rng.uniform(0.1, 0.3)), rot(float(pick(100.0, 10000.0, 1e6)), dims), int(rng.integers(2, 90)), ff))
+        else:
+            layers.append(latent2(*sizes, pick(None, 16, 40, 96), float(rng.uniform(0.1, 0.3)), rot(float(pick(500.0, 5e5)), dims, scaling), ff))
+    for i in range(len(layers)):
+        if rng.random() < 0.4:
+            layers.append(again(layers[i], i))
+    order = rng.permutation(len(layers)).tolist()              # any order: a layer may name one that runs after it
+    moved = []
+    for new, old in enumerate(order):
+        layer = json.loads(json.dumps(layers[old]))
+        if "weights_of" in layer:
+            layer["weights_of"] = order.index(layer["weights_of"])
+        moved.append(layer)
+    return config(int(rng.integers(40, 300)), pick(48, 64, 100, 136, 192), float(rng.uniform(0.2, 2.0)), pick(1e-5, 1e-6), moved)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("seed", range(8))
+def test_configurations_drawn_at_random_in_mixed_batches(tmp_path, seed, dtype):
+    from runtime.engine.replay import replay
+    cfg = random_config(seed)
+    folder = write_folder(tmp_path / "model", cfg, 100 + seed)
+    trace, seqs = mixed(cfg["vocab"], seed=30 + seed, lengths=(70, 33, 120, 9, 64, 97))
+    done = []
+    runner = replay(folder, dtype, tmp_path / "out", trace.peak, trace.lines(), echo=done.append, execution="graph" if seed % 2 else "eager")
+    assert done == [f"done {i}" for i in range(len(trace.steps))]
+    runner.cache.check()
+    trace.check(folder, tmp_path / "out", dtype, cfg["vocab"], seqs, plain=plain_logits)
