@@ -1,7 +1,7 @@
 """The Ditazen decoder as a list of parts chosen by DitazenConfig, layer by layer: pre-norm layers with centred norms
 (a weight, no bias), whose mixer is latent attention (two kinds: queries from one projection, split-half rotary pairs and
-a sliding window; or queries through a normed latent, neighbouring pairs with scaled frequencies, and every earlier
-key) or the gated delta rule, and whose feed-forward, if any, is one matrix up, gelu, one matrix down.  The logits are
+a sliding window; or queries through a normed latent, neighbouring pairs with scaled frequencies, and all keys
+up to its own) or the gated delta rule, and whose feed-forward, if any, is one matrix up, gelu, one matrix down.  The logits are
 the embedding table times the normed last rows, times `logit_scale` (which the last norm's weight carries).  A layer
 that names another's weights is the same part run at a further place of the schedule, with a cache or state of its own.
 Tensor names: `embed`, `l<i>.norm1|norm2`, `l<i>.mix.*`, `l<i>.mlp.up|down`, `final.norm`.

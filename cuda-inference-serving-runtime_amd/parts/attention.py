@@ -212,7 +212,7 @@ class LatentAttention(Mixer):
     """Softmax attention whose keys and values are made from one latent a token (multi-head latent attention).
 
     Per token the cache holds c = rms(Wdkv h)[:rank] * w (the latent) and kr = rot(Wdkv h [rank:]) (a key part that
-    turns with the position, shared by all heads).  Head j's key is [Wuk_j c | kr], its value Wuv_j c, its query
+    turns with the position, one for every head).  Head j's key is [Wuk_j c | kr], its value Wuv_j c, its query
     [q_j | rot(qr_j)] with `dim` plain and `rot_dim` turning coordinates; score = (q_j . Wuk_j c + rot(qr_j) . kr) scale,
     softmax over the visible keys (all earlier ones, or the last `window`).  Queries come from one projection, or with
     `q_rank` through a normed latent of their own: q = Wuq (rms(Wdq h) wq).  With `head_gate` a head's result is

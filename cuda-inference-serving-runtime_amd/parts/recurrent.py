@@ -171,7 +171,7 @@ class StateSpaceDuality(Mixer):
 class GatedDeltaRule(Mixer):
     """The gated delta rule.  `kv_heads` heads of q and k (`dim` each) serve `heads` heads of v (`vdim` each), head j
     using q/k head j // (heads / kv_heads).  `names`: the tensors' names under `name`; the convolutions' taps are
-    `<projection>.conv`, [channels, taps], the last column the current token's."""
+    `<projection>.conv`, [channels, taps]; tap n - 1 weighs the newest input."""
 
     NAMES = {"q": "q", "k": "k", "v": "v", "write": "b", "decay": "a", "dt_bias": "dt_bias", "a_log": "A_log", "gate": "g",
              "norm": "norm", "o": "o", "conv": "conv"}

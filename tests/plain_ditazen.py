@@ -107,8 +107,8 @@ def visible(T, window):
 
 
 def latent_attention(h, w, p, m, eps, second):
-    """`second` False: queries from one projection, rotate-half pairs, a sliding window (mask.size).
-    True: queries through a normed latent, interleaved pairs with scaled frequencies, every earlier key."""
+    """`second` False: queries from one projection, pairs (i, i + dims/2), the last mask.size keys.
+    True: queries through a normed latent, pairs (2i, 2i + 1) with scaled frequencies, all keys up to the query's own."""
     T = h.shape[0]
     H, D, R, V, r = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
     pos = np.arange(T)
@@ -138,7 +138,7 @@ def latent_attention(h, w, p, m, eps, second):
 # -- gated delta rule -------------------------------------------------------------------------------------------
 
 def causal_conv(x, taps):
-    """y[t, c] = sum_j taps[c, j] x[t - (n - 1) + j, c]: the last column is the current token's, zeros before the start."""
+    """y[t, c] = sum_j taps[c, j] x[t - (n - 1) + j, c]: tap n - 1 weighs x[t], and x is zero before row 0."""
     x, taps = np.asarray(x, np.float64), np.asarray(taps, np.float64)
     n = taps.shape[1]
     padded = np.concatenate([np.zeros((n - 1, x.shape[1])), x])
@@ -150,7 +150,7 @@ def unit(x):
 
 
 def delta_scan(q, k, v, beta, g):
-    """One head.  q, k [T, D]; v [T, V]; beta, g [T].  S [D, V] starts at zero."""
+    """One head.  q, k [T, D]; v [T, V]; beta, g [T].  S [D, V] is zero before the first row."""
     T, V = v.shape
     S = np.zeros((k.shape[1], V))
     out = np.zeros((T, V))

@@ -172,7 +172,7 @@ def test_unit_vectors_a_head():
     from runtime.kernels import ops
     rng = np.random.default_rng(3)
     x = rng.standard_normal((6, 4 + 3 * 10))
-    x[2, 4:14] = 0.0                                        # a head of zeros stays zero (eps inside the root)
+    x[2, 4:14] = 0.0                                        # a head of zeros stays zero (the root is of the sum plus eps)
     t = dev(x)
     ops.unit_heads(t[:, 4:], 3, 10, scale=0.5)
     got = host(t)
