@@ -568,7 +568,8 @@ def _skinny_ok(a, w):
 def _norm_args(x, norm, k):
     """(weight pointer, eps, rows pointer, number of output rows) for a fused RMSNorm prologue."""
     weight, eps, rows = norm
-    _dev(x, "x", torch.float32)
+    if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dtype != torch.float32 or x.dim() != 2 or x.stride(1) != 1:
+        raise KernelError("fused norm: expected float GPU rows with unit column stride (a view of wider rows will do)")
     if x.shape[1] != k or x.stride(0) % 8 or x.data_ptr() % 16:
         raise KernelError("fused norm: the residual rows must be 32-byte aligned floats of the product's inner size")
     wp = _dev(weight, "norm weight", torch.float32, (k,))

@@ -304,9 +304,15 @@ class LatentAttention(Mixer):
         small = ops.gemm(h, self.w_small, ctx.buffer("lat.small", (T, self.w_small.shape[0]), torch.float32), scratch=ctx.scratch)
         first = 0
         if self.q_rank is not None:
-            cq = ops.rms_slice(small[:, :self.q_size], self.q_weight, ctx.buffer("lat.cq", (T, self.q_size), ctx.dtype), self.eps)
-            h, first = cq, self.q_size
-        q = ops.gemm(h, self.w_q, ctx.buffer("lat.q", (T, nh * (D + R)), ctx.dtype), scratch=ctx.scratch)
+            first = self.q_size
+        q = ctx.buffer("lat.q", (T, nh * (D + R)), ctx.dtype)
+        if self.q_rank is not None and ops.fused_norm_ok(small[:, :first], self.w_q, T):
+            # few rows: the query latent's norm rides in the product that reads it
+            ops.gemm_normed(small[:, :first], (self.q_weight, self.eps, None), self.w_q, q)
+        else:
+            if self.q_rank is not None:
+                h = ops.rms_slice(small[:, :first], self.q_weight, ctx.buffer("lat.cq", (T, first), ctx.dtype), self.eps)
+            ops.gemm(h, self.w_q, q, scratch=ctx.scratch)
         qa = ctx.buffer("lat.qa", (T, nh * pad), ctx.dtype)
         ops.latent_keys(small[:, first:first + r + R], self.kv_weight, q, qa, kcache, vcache, ctx.positions, view.slots, cos, sin,
                         nh, D, R, r, pad, view.page_size, self.eps, interleaved=self.position.pairing == "interleaved")
