@@ -57,6 +57,7 @@ _A = [latent(3, 16, 8, 24, 40, 0.2, rot(10000.0, 8), 21, mlp(96)),
 _S = [latent(4, 8, 16, 16, 24, 0.35, rot(1000.0, 16), 19, mlp(64)),
       delta(2, 2, 24, 16, 4),
       latent2(2, 16, 8, 24, 32, 16, 0.4, rot(20000.0, 8, (4.0, 32, 8.0, 1.0)), mlp(48))]
+_F = latent2(3, 16, 8, 16, 24, 32, 0.45, rot(8000.0, 8, (4.0, 128, 16.0, 1.0)), mlp(56))
 CONFIGS = {
     # every kind of layer, then two of them once more with the first ones' weights; a layer without a feed-forward
     "a": config(131, 64, 0.3, 1e-5, _A + [again(_A[1], 1), again(_A[0], 0)]),
@@ -75,10 +76,14 @@ CONFIGS = {
         latent(20, 8, 8, 8, 16, 0.3, rot(500.0, 8), 33, mlp(40)),
         latent2(3, 8, 8, 16, 296, 16, 0.06, rot(3000.0, 8, (2.0, 64, 8.0, 2.0))),
         delta(2, 1, 256, 8, 2)]),
+    # only attention over all keys (no window, no state): what the last rows know of the first ones they know through
+    # far keys alone; drawn sharp
+    "f": config(89, 40, 0.9, 1e-5, [_F, again(_F, 0)]),
     # no layer keeps pages: the cache manager has state slots only
     "d": config(53, 40, 1.0, 1e-5, [delta(4, 1, 8, 12, 2, mlp(48)), delta(3, 3, 20, 8, 5)]),
 }
-SEEDS = {"a": 21, "b": 22, "s": 23, "d": 24, "w": 25}
+SEEDS = {"a": 21, "b": 22, "s": 23, "d": 24, "w": 25, "f": 26}
+SHARP = ("s", "f")
 FILE_Q_RANK = 28       # the query latent of configuration "b", which config.json does not give
 
 

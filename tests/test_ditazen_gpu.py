@@ -11,7 +11,7 @@ import torch
 
 import plain_ditazen as P
 from conftest import assert_close, random_tokens
-from ditazen_models import CONFIGS, SEEDS, plain_logits, write_folder
+from ditazen_models import CONFIGS, SEEDS, SHARP, plain_logits, write_folder
 from trace_tools import Trace
 
 pytestmark = pytest.mark.gpu
@@ -23,7 +23,7 @@ TORCH = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 @pytest.fixture(scope="module")
 def folders(tmp_path_factory):
     base = tmp_path_factory.mktemp("ditazen")
-    return {name: write_folder(base / name, CONFIGS[name], SEEDS[name], sharp=name == "s") for name in CONFIGS}
+    return {name: write_folder(base / name, CONFIGS[name], SEEDS[name], sharp=name in SHARP) for name in CONFIGS}
 
 
 def dev(a, dtype=torch.float32):
@@ -407,6 +407,27 @@ def test_far_keys_page_borders_the_windows_edge_and_old_state_in_a_model_drawn_s
     assert_close(got[:3], want[:3], dtype, "the first tokens")
     if dtype == "float32":
         assert np.abs(got - want).max() / scale < bound       # every row, also those at the window's edge
+    runner.cache.check()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_keys_hundreds_of_tokens_back_through_attention_alone(folders, dtype):
+    """A model of attention over all keys only, drawn sharp: the last rows know the first tokens through far keys and
+    nothing else.  A prompt cut inside a page, then tokens one by one across page borders."""
+    from runtime.engine import StepEntry
+    name = "f"
+    cfg, w = P.read_folder(folders[name])
+    tokens = random_tokens(12, 430, cfg["vocab"])
+    want = plain_logits(folders[name], tokens)
+    late = P.forward(cfg, w, tokens[300:])
+    assert np.linalg.norm(late[-60:] - want[-60:]) / np.linalg.norm(want[-60:]) > 3 * 0.04, "the first 300 tokens do not reach the last 60"
+    runner = make_runner(folders[name], dtype, pages=28)
+    runner.create("f")
+    got = [runner.step([StepEntry("f", tokens[:153], list(range(153)))]).cpu().numpy(),
+           runner.step([StepEntry("f", tokens[153:390], list(range(237)))]).cpu().numpy()]
+    got += [runner.step([StepEntry("f", [t], [0])]).cpu().numpy() for t in tokens[390:]]
+    assert_close(np.concatenate(got), want, dtype, "far keys")
+    assert_close(np.concatenate(got)[-40:], want[-40:], dtype, "the last rows")
     runner.cache.check()
 
 

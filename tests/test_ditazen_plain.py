@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 import plain_ditazen as P
-from ditazen_models import CONFIGS, SEEDS, FILE_Q_RANK, tensor_shapes, write_folder
+from ditazen_models import CONFIGS, SEEDS, SHARP, FILE_Q_RANK, tensor_shapes, write_folder
 
 
 def test_delta_rule_writes_what_it_is_asked_to_remember():
@@ -112,7 +112,7 @@ def test_window_and_latent_attention_by_hand():
 
 @pytest.mark.parametrize("name", sorted(CONFIGS))
 def test_logits_depend_on_earlier_tokens_only(tmp_path, name):
-    cfg, w = P.read_folder(write_folder(tmp_path, CONFIGS[name], SEEDS[name], sharp=name == "s"))
+    cfg, w = P.read_folder(write_folder(tmp_path, CONFIGS[name], SEEDS[name], sharp=name in SHARP))
     tokens = np.random.default_rng(1).integers(0, cfg["vocab"], 40).tolist()
     full = P.forward(cfg, w, tokens)
     np.testing.assert_allclose(P.forward(cfg, w, tokens[:23]), full[:23], rtol=1e-9, atol=1e-9)
