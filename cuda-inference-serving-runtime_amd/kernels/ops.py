@@ -1032,8 +1032,9 @@ def heads_product(a, a_head, w, out, out_head, gate=None):
     unit column stride; w [heads, N, K] contiguous."""
     heads, n, k = w.shape
     rows = a.shape[0]
-    if a.dtype != w.dtype or out.dtype != w.dtype or a.stride(1) != 1 or out.stride(1) != 1 or out.shape[0] != rows:
-        raise KernelError("heads_product: operands of one dtype with contiguous rows")
+    if (not a.is_cuda or not out.is_cuda or a.dim() != 2 or out.dim() != 2 or a.dtype != w.dtype or out.dtype != w.dtype
+            or a.stride(1) != 1 or out.stride(1) != 1 or out.shape[0] != rows):
+        raise KernelError("heads_product: GPU operands of one dtype with contiguous rows")
     if a.shape[1] < (heads - 1) * a_head + k or out.shape[1] < (heads - 1) * out_head + n:
         raise KernelError("heads_product: rows too short for their heads")
     gp, ldg = (None, 0) if gate is None else _rows_of(gate, "gate", heads)
