@@ -58,9 +58,12 @@ extern "C" int cisr_linear_scan(const float* q, int ldq, const float* k, int ldk
 // out[t * channels + ch] = silu(bias[ch] + sum_j w[ch * taps + j] * input(t - (taps - 1) + j)).
 // Index channels + h, h < heads (if heads > 0): step[t * heads + h] = softplus(in[t * ld + dt_first + h] + dt_bias[h]),
 // decay[t * heads + h] = exp(-exp(a_log[h]) * step).
+// SINGLE: every segment has one row (a step of single tokens), so the thread of a (row, channel) is the only one that
+// reads that channel of its request's state, and it moves the state on itself: no second launch.
+template <bool SINGLE>
 __global__ void __launch_bounds__(256)
 conv_silu_kernel(const float* __restrict__ in, int ld, int first, const float* __restrict__ w, const float* __restrict__ bias,
-                 const float* __restrict__ conv_state, long long slot_stride, float* __restrict__ out,
+                 float* conv_state, long long slot_stride, float* __restrict__ out,
                  const int* __restrict__ seg_of_row, const int* __restrict__ seg_start, const int* __restrict__ state_slots,
                  int channels, int taps, int heads, int dt_first, const float* __restrict__ dt_bias,
                  const float* __restrict__ a_log, float* __restrict__ step, float* __restrict__ decay) {
@@ -77,12 +80,13 @@ conv_silu_kernel(const float* __restrict__ in, int ld, int first, const float* _
         return;
     }
     const int rel = t - seg_start[seg];
-    const float* st = conv_state + (long long)state_slots[seg] * slot_stride;
+    float* st = conv_state + (long long)state_slots[seg] * slot_stride;
     float y = bias ? bias[idx] : 0.f;
     for (int j = 0; j < taps; ++j) {
         const int src = rel - (taps - 1) + j;
         const float x = src >= 0 ? in[(size_t)(t - rel + src) * ld + first + idx] : st[(size_t)(taps - 1 + src) * channels + idx];
         y += w[(size_t)idx * taps + j] * x;
+        if (SINGLE && j > 0) st[(size_t)(j - 1) * channels + idx] = x;     // (input j of this row is input j - 1 of the next)
     }
     out[(size_t)t * channels + idx] = y / (1.0f + expf(-y));
 }
@@ -113,10 +117,16 @@ extern "C" int cisr_conv_silu(const float* in, int ld, int first, const float* w
                               long long slot_stride, float* out, const int* seg_of_row, const int* seg_start,
                               const int* state_slots, int rows, int segments, int channels, int taps, int heads,
                               int dt_first, const float* dt_bias, const float* a_log, float* step, float* decay,
-                              hipStream_t stream) {
+                              int single_rows, hipStream_t stream) {
     if (rows <= 0 || segments <= 0) return 0;
     if (channels <= 0 || taps < 1 || taps > MAX_TAPS || heads < 0 || segments > 65535) return (int)hipErrorInvalidValue;
-    conv_silu_kernel<<<dim3(rows, (channels + heads + 255) / 256), 256, 0, stream>>>(in, ld, first, w, bias, conv_state, slot_stride,
+    const dim3 grid(rows, (channels + heads + 255) / 256);
+    if (single_rows) {       // `single_rows`: the caller knows that no segment has more than one row
+        conv_silu_kernel<true><<<grid, 256, 0, stream>>>(in, ld, first, w, bias, conv_state, slot_stride,
+            out, seg_of_row, seg_start, state_slots, channels, taps, heads, dt_first, dt_bias, a_log, step, decay);
+        return CISR_LAUNCH_CHECK();
+    }
+    conv_silu_kernel<false><<<grid, 256, 0, stream>>>(in, ld, first, w, bias, conv_state, slot_stride,
         out, seg_of_row, seg_start, state_slots, channels, taps, heads, dt_first, dt_bias, a_log, step, decay);
     int err = CISR_LAUNCH_CHECK();
     if (err || taps == 1) return err;

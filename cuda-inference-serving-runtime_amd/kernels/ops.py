@@ -1099,7 +1099,7 @@ def _rec():
         p, i, f, ll = C.c_void_p, C.c_int, C.c_float, C.c_longlong
         sig = {
             "cisr_linear_scan": [p, i, p, i, p, i, p, i, i, p, i, p, i, p, ll, p, p, i, i, i, i, i, f, i, i, i, p, p, p],
-            "cisr_conv_silu": [p, i, i, p, p, p, ll, p, p, p, p, i, i, i, i, i, i, p, p, p, p, p],
+            "cisr_conv_silu": [p, i, i, p, p, p, ll, p, p, p, p, i, i, i, i, i, i, p, p, p, p, i, p],
             "cisr_decay_gate": [p, i, p, p, i, i, f, p],
             "cisr_decay_gate_low_rank": [p, i, i, p, p, p, i, i, f, p],
             "cisr_group_norm_gate": [p, p, i, p, i, p, i, p, i, p, i, i, i, f, i, i, p],
@@ -1193,12 +1193,14 @@ def linear_scan(q, k, v, decay, out, state, seg_start, state_slots, heads, rows_
     return out
 
 
-def conv_silu(x, taps_weight, bias, conv_state, out, seg_of_row, seg_start, state_slots, gates=None):
+def conv_silu(x, taps_weight, bias, conv_state, out, seg_of_row, seg_start, state_slots, gates=None, single_rows=False):
     """out[t, c] = silu(bias[c] + sum_j w[c, j] input(t - (K - 1) + j)[c]) over the rows of each segment, the K - 1 inputs
     before a segment's first row taken from its state slot, which then moves on to the last K - 1 inputs.
     x float view [T, channels]; taps_weight float [channels, K]; conv_state float view [slots, >= (K - 1) * channels].
     `gates` = (dt view [T, heads], dt_bias [heads], a_log [heads], step out [T, heads], decay out [T, heads]):
-    step = softplus(dt + dt_bias), decay = exp(-exp(a_log) step), made by the same launch."""
+    step = softplus(dt + dt_bias), decay = exp(-exp(a_log) step), made by the same launch.
+    `single_rows`: the caller vouches that no segment has more than one row (a step of single tokens); the state then
+    moves on in the same launch instead of a second one."""
     T, channels = x.shape
     K = taps_weight.shape[1]
     segments = state_slots.shape[0]
@@ -1221,7 +1223,7 @@ def conv_silu(x, taps_weight, bias, conv_state, out, seg_of_row, seg_start, stat
                                  _dev(seg_of_row, "seg_of_row", torch.int32, (T,)),
                                  _dev(seg_start, "seg_start", torch.int32, (segments + 1,)),
                                  _dev(state_slots, "state_slots", torch.int32, (segments,)), T, segments, channels, K, heads,
-                                 dt_first, bp2, alp, stp, dcp, _stream()), "conv_silu")
+                                 dt_first, bp2, alp, stp, dcp, int(bool(single_rows)), _stream()), "conv_silu")
     return out
 
 

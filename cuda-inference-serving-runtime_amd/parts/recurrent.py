@@ -155,7 +155,8 @@ class StateSpaceDuality(Mixer):
         xbc = ctx.buffer("ssd.xbc", (T, ch), torch.float32)
         step, decay = ctx.buffer("ssd.step", (T, nh), torch.float32), ctx.buffer("ssd.decay", (T, nh), torch.float32)
         ops.conv_silu(proj[:, inner:inner + ch], self.conv, self.conv_bias, state[:, heads_state:], xbc, ctx.seg_of_row,
-                      ctx.seg_start, ctx.state_slots, gates=(proj[:, inner + ch:], self.dt_bias, self.a_log, step, decay))
+                      ctx.seg_start, ctx.state_slots, gates=(proj[:, inner + ch:], self.dt_bias, self.a_log, step, decay),
+                      single_rows=ctx.decode_only)
         y = ctx.buffer("ssd.o", (T, inner), torch.float32)
         _scan(ctx, "ssd", xbc[:, inner + GN:], xbc[:, inner:inner + GN], xbc[:, :inner], decay, y, state,
               nh, self.state, self.vdim, share=nh // self.groups, step=step)
@@ -234,7 +235,7 @@ class GatedDeltaRule(Mixer):
         qkv = ctx.buffer("delta.qkv", (T, ch), torch.float32)
         step, decay = ctx.buffer("delta.step", (T, nh), torch.float32), ctx.buffer("delta.decay", (T, nh), torch.float32)
         ops.conv_silu(proj[:, :ch], self.conv, None, state[:, heads_state:], qkv, ctx.seg_of_row, ctx.seg_start, ctx.state_slots,
-                      gates=(proj[:, ch:ch + nh], self.dt_bias, self.a_log, step, decay))
+                      gates=(proj[:, ch:ch + nh], self.dt_bias, self.a_log, step, decay), single_rows=ctx.decode_only)
         ops.unit_heads(qkv[:, :2 * qk], 2 * self.kv_heads, self.dim, eps=self.unit_eps)
         o = ctx.buffer("delta.o", (T, inner), torch.float32)
         ops.delta_scan(qkv[:, :qk], qkv[:, qk:2 * qk], qkv[:, 2 * qk:], decay, proj[:, ch + nh:ch + 2 * nh], o, state,

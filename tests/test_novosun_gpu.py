@@ -128,7 +128,7 @@ def test_linear_scan_in_pieces_side_by_side_equals_the_scan_in_order(heads, shar
 def test_short_convolution_carries_its_last_inputs_across_portions_of_any_size(channels, taps, heads):
     from runtime.kernels import ops
     rng = np.random.default_rng(channels)
-    n = {"a": 23, "b": 9}
+    n = {"a": 23, "b": 10}
     width = 4 + channels + heads
     x = {k: rng.standard_normal((v, width)) for k, v in n.items()}
     w, b = rng.standard_normal((channels, taps)), rng.standard_normal(channels)
@@ -140,8 +140,9 @@ def test_short_convolution_carries_its_last_inputs_across_portions_of_any_size(c
     state[2, 11:].zero_()
     fed = {"a": 0, "b": 0}
     got = {"a": [], "b": []}
-    for portion in [{"a": 1, "b": 2}, {"a": 2}, {"b": 1, "a": 1}, {"a": 7, "b": 6}, {"a": 12}]:       # shorter than the taps, and longer
+    for portion in [{"a": 1, "b": 2}, {"a": 2}, {"b": 1, "a": 1}, {"a": 7, "b": 6}, {"a": 1}, {"a": 1, "b": 1}, {"a": 10}]:       # shorter than the taps, and longer
         keys = list(portion)
+        single = all(count == 1 for count in portion.values())        # steps of single tokens move the state on in the same launch
         rows = np.concatenate([x[k][fed[k]:fed[k] + portion[k]] for k in keys])
         starts = np.concatenate(([0], np.cumsum([portion[k] for k in keys])))
         seg_of_row = np.repeat(np.arange(len(keys)), [portion[k] for k in keys])
@@ -152,7 +153,7 @@ def test_short_convolution_carries_its_last_inputs_across_portions_of_any_size(c
             step, decay = torch.zeros((len(rows), heads), device=DEV), torch.zeros((len(rows), heads), device=DEV)
             gates = (full[:, 4 + channels:], dev(dt_bias), dev(a_log), step, decay)
         ops.conv_silu(full[:, 4:4 + channels], dev(w), dev(b), conv_state, out, ints(seg_of_row), ints(starts),
-                      ints([{"a": 2, "b": 0}[k] for k in keys]), gates=gates)
+                      ints([{"a": 2, "b": 0}[k] for k in keys]), gates=gates, single_rows=single)
         if heads:
             dt = P.softplus(rows[:, 4 + channels:] + dt_bias)
             close(step.cpu().numpy(), dt)
